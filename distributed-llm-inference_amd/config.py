@@ -25,8 +25,13 @@ class MixerSpec:
     the leading ``rot_dims`` entries of every head with optionally stretched frequencies, a per-head sink in the softmax
     denominator, softmax weights mixed across heads, sigmoid output gate), ``"time_mix"`` (recurrence with a per-token,
     per-channel decay from a low-rank projection, a bonus for the current token and a ``[D, D]`` state per head; all five
-    projections read their own blend of the token's and the previous token's input) or ``"parallel"`` (the mixers in
-    ``parts`` read the same input; their outputs are summed with the weights ``part_scales``)."""
+    projections read their own blend of the token's and the previous token's input), ``"parallel"`` (the mixers in
+    ``parts`` read the same input; their outputs are summed with the weights ``part_scales``), ``"gated_attention"`` (causal
+    grouped-query softmax attention without positions: q / k normalised over the whole projection, one sigmoid output gate
+    per head; ``kv_from`` ≥ 0: the layer has no key / value projections and reads that layer's cache) or ``"retention"``
+    (linear attention with a per-head decay and no activation or denominator: half-split rotation of the leading
+    ``rot_dims`` entries of q and k, keys scaled by ``dim**-0.5``, a ``[D, Dv]`` state per head, per-head unit RMS and a
+    silu gate behind it)."""
     kind: str
     heads: int
     dim: int                            # per-head query / key size (latent attention: the unrotated part)
@@ -49,16 +54,19 @@ class MixerSpec:
     top: int = 0                        # moe: experts per token
     router_scale: float = 1.0           # moe: multiplies the chosen experts' scores
     shared_ff: int = 0                  # moe: inner width of the expert every token takes (0: none)
+    kv_from: int = -1                   # gated attention: index of the layer whose cached keys / values this layer reads (-1: its own)
+    ff_act: str = "relu2"               # feed-forward activation: "relu2" | "gelu_tanh" (gated dense) | "silu" (gated experts)
+    router: str = "sigmoid"             # moe: "sigmoid" (scores, not renormalised) | "softmax" (biased logits, softmax over the chosen)
 
     @property
     def stateful(self) -> bool:
-        return self.kind in ("lightning", "time_mix") or any(p.stateful for p in self.parts)
+        return self.kind in ("lightning", "time_mix", "retention") or any(p.stateful for p in self.parts)
 
     @property
     def cache_row(self) -> tuple:
         """Widths of the per-token rows this mixer keeps in the paged cache: ``(key row, value row)``; a latent mixer keeps
         one row (latent | rotated key) that serves as both; a recurrent one keeps none."""
-        if self.kind in ("attention", "sink_attention"):
+        if self.kind in ("attention", "sink_attention") or (self.kind == "gated_attention" and self.kv_from < 0):
             return self.kv_heads * self.dim, self.kv_heads * self.vdim
         if self.kind == "parallel":
             return tuple(sum(w) for w in zip(*(p.cache_row for p in self.parts)))
@@ -70,7 +78,7 @@ class MixerSpec:
     def state_shape(self) -> tuple:
         if self.kind == "parallel":
             return next((p.state_shape for p in self.parts if p.state_shape), ())
-        return (self.heads, self.dim, self.vdim) if self.kind in ("lightning", "time_mix") else ()
+        return (self.heads, self.dim, self.vdim) if self.kind in ("lightning", "time_mix", "retention") else ()
 
 
 @dataclass
@@ -103,6 +111,12 @@ class ModelConfig:
     loop: Optional[tuple] = None
     residual_mult: float = 1.0          # a sublayer's normalised output enters the stream times this
     logit_softcap: float = 0.0          # logits ← cap · tanh(logits / cap); 0: off
+    # hyper-connected stacks (arch "sevelorn"): ``streams`` copies of the residual stream that every sublayer reads as a
+    # weighted sum and updates through a mixing matrix (0: one plain stream); ``conv_taps``: taps of the causal per-channel
+    # convolution added to every mixer's input (0: none); ``embed_scale`` multiplies the embedding rows
+    streams: int = 0
+    conv_taps: int = 0
+    embed_scale: float = 1.0
 
     @property
     def layer_runs(self) -> tuple:
@@ -127,6 +141,8 @@ class ModelConfig:
 
     def param_count(self) -> int:
         h, i, v, l = self.hidden_size, self.intermediate_size, self.vocab_size, self.num_layers
+        if self.arch == "sevelorn":
+            return 2 * v * h + h + sum(_hyper_layer_params(m, h, self.streams, self.conv_taps) for m in self.layer_specs)
         if self.layer_specs:
             tot = 2 * v * h + 2 * h
             for m in self.layer_specs:
@@ -163,6 +179,20 @@ def _parallel_layer_params(m: MixerSpec, h: int) -> int:
             tot += 5 * h + 5 * c * h + p.lora * (h + c) + 3 * c
     if m.ff:
         tot += m.experts * (2 * h * m.ff + h) + (2 * h * m.shared_ff + h if m.shared_ff else 0)
+    return tot
+
+
+def _hyper_layer_params(m: MixerSpec, h: int, streams: int, taps: int) -> int:
+    """Parameters of one hyper-connected layer (norms, stream weights, input convolution, mixer, feed-forward)."""
+    hc = (2 * streams + streams * streams) if streams else 0
+    tot = h + hc + taps * h
+    if m.kind == "gated_attention":
+        kv = 0 if m.kv_from >= 0 else h * m.kv_heads * (m.dim + m.vdim) + m.kv_heads * m.dim
+        tot += h * m.heads * m.dim + m.heads * m.dim + kv + m.heads * h + m.heads * m.vdim * h
+    else:
+        tot += h * m.heads * (2 * m.dim + 2 * m.vdim) + m.heads * m.vdim * h
+    if m.ff:
+        tot += h + hc + (m.experts * 3 * h * m.ff + m.experts * (h + 1) if m.ff_kind == "moe" else 3 * h * m.ff)
     return tot
 
 
@@ -237,7 +267,63 @@ def vibunex_config(cfg: dict, name: str = "vibunex", dtype: str = "bfloat16", sh
                        residual_mult=float(cfg.get("residual_mult", 1.0)))
 
 
-_CONFIG_READERS = {"Rodelix": rodelix_config, "Vibunex": vibunex_config}
+def _sevelorn_spec(entry: dict, index: int, layers: list) -> MixerSpec:
+    m, mlp = entry["mixer"], entry.get("mlp")
+    kind = entry["type"]
+    ff = {}
+    if mlp:
+        if mlp.get("kind") == "dense":
+            ff = dict(ff=int(mlp["ff"]), ff_kind="dense", ff_act="gelu_tanh")
+        elif mlp.get("kind") == "moe":
+            r = mlp["router"]
+            ff = dict(ff=int(mlp["expert"]["ff"]), ff_kind="moe", ff_act="silu", router="softmax", experts=int(r["experts"]),
+                      top=int(r["top"]))
+            if not 1 <= ff["top"] <= ff["experts"]:
+                raise ValueError(f"layer {index}: {ff['top']} of {ff['experts']} experts")
+        else:
+            raise ValueError(f"layer {index}: unknown feed-forward kind {mlp.get('kind')!r}")
+    common = dict(heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), **ff)
+    if kind == "attention":
+        src = m.get("kv_from")
+        spec = MixerSpec(kind="gated_attention", kv_heads=int(m["kv_heads"]), scale=float(m["scale"]),
+                         kv_from=-1 if src is None else int(src), **common)
+        if spec.heads % spec.kv_heads:
+            raise ValueError(f"layer {index}: {spec.heads} query heads over {spec.kv_heads} key/value heads")
+        if src is not None:
+            if not 0 <= spec.kv_from < index:
+                raise ValueError(f"layer {index}: keys / values from layer {src}, which does not run before it")
+            o = layers[spec.kv_from]
+            om = o["mixer"]
+            if o["type"] != "attention" or om.get("kv_from") is not None:
+                raise ValueError(f"layer {index}: layer {src} keeps no keys / values of its own")
+            if (int(om["kv_heads"]), int(om["dim"]), int(om["vdim"])) != (spec.kv_heads, spec.dim, spec.vdim):
+                raise ValueError(f"layer {index}: key / value sizes differ from those of layer {src}")
+        return spec
+    if kind == "retention":
+        rot = m.get("rot") or {}
+        spec = MixerSpec(kind="retention", decay=tuple(float(d) for d in m["decay"]), rot_base=float(rot.get("base", 10000.0)),
+                         rot_dims=int(rot.get("dims", 0)), **common)
+        if len(spec.decay) != spec.heads:
+            raise ValueError(f"layer {index}: {len(spec.decay)} decays for {spec.heads} heads")
+        if spec.rot_dims % 2 or spec.rot_dims > spec.dim:
+            raise ValueError(f"layer {index}: {spec.rot_dims} rotated entries of {spec.dim}")
+        return spec
+    raise ValueError(f"layer {index}: unknown mixer type {kind!r}")
+
+
+def sevelorn_config(cfg: dict, name: str = "sevelorn", dtype: str = "bfloat16") -> ModelConfig:
+    """``ModelConfig`` of a Sevelorn checkpoint from the dict its ``config.json`` holds."""
+    specs = tuple(_sevelorn_spec(e, i, cfg["layers"]) for i, e in enumerate(cfg["layers"]))
+    att = next((s for s in specs if s.kind == "gated_attention"), specs[0])
+    return ModelConfig(name=name, arch="sevelorn", vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]),
+                       intermediate_size=max([s.ff for s in specs] + [0]), num_layers=len(specs), num_heads=att.heads,
+                       num_kv_heads=max(att.kv_heads, 1), head_dim=att.dim, max_position=1 << 24,
+                       rms_eps=float(cfg["norm"]["eps"]), dtype=dtype, bos_token_id=0, eos_token_id=-1, layer_specs=specs,
+                       streams=int(cfg.get("streams") or 0), conv_taps=int((cfg.get("canon") or {}).get("taps", 0)),
+                       embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)))
+
+
+_CONFIG_READERS = {"Rodelix": rodelix_config, "Vibunex": vibunex_config, "Sevelorn": sevelorn_config}
 
 
 def safetensors_shapes(path: str) -> dict:
@@ -356,6 +442,18 @@ MODEL_PRESETS: dict[str, ModelConfig] = {
                        "right": {"heads": 3, "dim": 16, "lora": 4}},
              "mlp": None}]},
         name="tiny-vibunex", dtype="float32"),
+    # hyper-connected streams, input convolution, gated attention (one layer on another's keys / values), retention,
+    # dense and routed gated feed-forwards
+    "tiny-sevelorn": sevelorn_config({
+        "vocab": 352, "width": 80, "streams": 2, "canon": {"taps": 4}, "embedding": {"scale": 2.0}, "norm": {"eps": 1e-5},
+        "layers": [
+            {"type": "retention", "mlp": {"kind": "dense", "ff": 112},
+             "mixer": {"heads": 3, "dim": 16, "vdim": 32, "decay": [0.9, 0.97, 0.995], "rot": {"base": 5000.0, "dims": 8}}},
+            {"type": "attention", "mlp": {"kind": "moe", "expert": {"ff": 48}, "router": {"experts": 5, "top": 2}},
+             "mixer": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 24, "scale": 0.3}},
+            {"type": "attention", "mlp": None,
+             "mixer": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 24, "scale": 0.2, "kv_from": 1}}]},
+        name="tiny-sevelorn", dtype="float32"),
     "tiny-opt": ModelConfig(name="tiny-opt", arch="opt", vocab_size=512, hidden_size=64,
                             intermediate_size=128, num_layers=2, num_heads=4, num_kv_heads=4,
                             head_dim=16, max_position=512, pos_offset=2, tie_embeddings=True,

@@ -19,10 +19,11 @@ from .layers import random_full_tensor
 from .llama import LlamaForCausalLM
 from .opt import OPTForCausalLM
 from .rodelix import RodelixForCausalLM
+from .sevelorn import SevelornForCausalLM
 from .vibunex import VibunexForCausalLM
 
 _ARCH = {"llama": LlamaForCausalLM, "mixtral": LlamaForCausalLM, "opt": OPTForCausalLM, "rodelix": RodelixForCausalLM,
-         "vibunex": VibunexForCausalLM}
+         "vibunex": VibunexForCausalLM, "sevelorn": SevelornForCausalLM}
 
 
 def torch_dtype(name: str) -> torch.dtype:

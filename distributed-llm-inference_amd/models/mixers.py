@@ -20,6 +20,16 @@ cache)`` that serves prefill chunks and decode rows of a mixed step alike:
 ``GatedParallelLayer`` runs a mixer and a feed-forward on two scalar-gain RMS norms of the same stream and adds
 both, each through a sigmoid gate computed from its own input: ``x += m · (g1 ⊙ mixer(n1) + g2 ⊙ ff(n2))``.
 
+* ``GatedAttention`` – causal grouped-query attention without positions: whole-projection q / k norm, one sigmoid output
+  gate per head; optionally without key / value projections of its own, on another layer's cache;
+* ``Retention`` – linear attention with a per-head decay and no activation: rotated q / k, scaled keys, a ``[D, Dv]``
+  fp32 state per head, per-head unit RMS and a silu gate behind it.
+
+``GatedDenseFF`` (``W_down (act(W_gate h) ⊙ W_up h)``) and ``SoftmaxRoutedFF`` (experts of that form behind a biased
+fp32 router, softmax over the chosen logits) are the feed-forwards of ``HyperLayer``, which keeps several copies of the
+fp32 stream: every sublayer reads a weighted sum of them through an RMS norm (the mixer also through a short causal
+convolution over time) and writes back through a mixing matrix.
+
 ``MixerLayer`` wraps one of the first three (and an optional dense feed-forward) in the sandwich
 ``x += m · norm_b(sublayer(norm(x)))`` with token shift in front of the mixer.  The residual stream ``x`` is
 fp32; GEMM operands are the model dtype.  Tensor parallelism is not implemented for these stacks.
@@ -48,6 +58,7 @@ class LayerCache:
     v: Optional[torch.Tensor] = None
     state: Optional[torch.Tensor] = None
     shift: Optional[torch.Tensor] = None
+    owns_pages: bool = True             # False: ``k`` / ``v`` are another layer's pages (a mixer without keys / values of its own)
 
 
 def _param(shape, ctx, device) -> Weight:
@@ -289,7 +300,83 @@ class DualMixer(nn.Module):
         return [left, self.right(h, meta, cache)], extra
 
 
-MIXERS = {"attention": WindowAttention, "latent_attention": LatentAttention, "lightning": LightningAttention,
+class GatedAttention(nn.Module):
+    """``spec.kv_from`` ≥ 0: no key / value projections; ``forward`` reads the pages it is handed (that layer's)."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, ctx: ParallelContext, dtype, device):
+        super().__init__()
+        self.s, self.eps = spec, eps
+        H, G, D, Dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+        assert H % G == 0, "query heads must be a multiple of the key/value heads"
+        self.own_kv = spec.kv_from < 0
+        Gp = G if self.own_kv else 0
+        self.cols = (H * D, Gp * D, Gp * Dv, H)                     # q | k | v | one output gate per head
+        self.qkvg = _matrix(sum(self.cols), width, ctx, dtype, device)
+        self.o = _matrix(width, H * Dv, ctx, dtype, device)
+        self.q_norm = _param((H * D,), ctx, device)
+        self.k_norm = _param((G * D,), ctx, device) if self.own_kv else None
+
+    def weights(self, p):
+        yield p + "qkvg", self.qkvg, "normal", [p + "q"] + ([p + "k", p + "v"] if self.own_kv else []) + [p + "g"]
+        yield p + "o", self.o, "normal", None
+        yield p + "q.norm", self.q_norm, "ones", None
+        if self.own_kv:
+            yield p + "k.norm", self.k_norm, "ones", None
+
+    def cache(self, num_blocks, num_slots, dtype, device) -> LayerCache:
+        s = self.s
+        if not self.own_kv:
+            return LayerCache(owns_pages=False)
+        return LayerCache(k=torch.zeros(num_blocks, KV_BLOCK_SIZE, s.kv_heads * s.dim, dtype=dtype, device=device),
+                          v=torch.zeros(num_blocks, KV_BLOCK_SIZE, s.kv_heads * s.vdim, dtype=dtype, device=device))
+
+    def forward(self, h, meta, cache: LayerCache):
+        s = self.s
+        H, G, D, Dv = s.heads, s.kv_heads, s.dim, s.vdim
+        T = h.shape[0]
+        nq, nk, nv, ng = self.cols
+        both = ops.linear(h, self.qkvg.data)
+        seqmix.wide_norm_rope_cache(both, self.q_norm.data, self.k_norm.data if self.own_kv else None, self.eps, meta.positions,
+                                    None, 1.0, 0, meta.slot_mapping, cache.k, cache.v, H, G if self.own_kv else 0, D, Dv)
+        out = torch.zeros(T, H, Dv, dtype=h.dtype, device=h.device)      # padding rows of a captured step stay zero
+        seqmix.token_attention(out, both[:, :nq].unflatten(1, (H, D)), None, cache.k, cache.v, meta, G, Dv, s.scale,
+                               gate=both[:, nq + nk + nv:])
+        return ops.linear(out.view(T, H * Dv), self.o.data)
+
+
+class Retention(nn.Module):
+    def __init__(self, spec: MixerSpec, width: int, eps: float, ctx: ParallelContext, dtype, device):
+        super().__init__()
+        self.s, self.eps = spec, eps
+        H, D, Dv = spec.heads, spec.dim, spec.vdim
+        assert len(spec.decay) == H, "one decay per head"
+        assert spec.rot_dims % 2 == 0 and spec.rot_dims <= D
+        self.qkvg = _matrix(2 * H * D + 2 * H * Dv, width, ctx, dtype, device)
+        self.o = _matrix(width, H * Dv, ctx, dtype, device)
+        self.register_buffer("decay", torch.tensor(spec.decay, dtype=torch.float32, device=device), persistent=False)
+        self.register_buffer("inv_freq", seqmix.rotary_inv_freq(spec.rot_base, spec.rot_dims, device) if spec.rot_dims else None,
+                             persistent=False)
+
+    def weights(self, p):
+        yield p + "qkvg", self.qkvg, "normal", [p + "q", p + "k", p + "v", p + "g"]
+        yield p + "o", self.o, "normal", None
+
+    def cache(self, num_blocks, num_slots, dtype, device) -> LayerCache:
+        s = self.s
+        return LayerCache(state=torch.zeros(num_slots, s.heads, s.dim, s.vdim, dtype=torch.float32, device=device))
+
+    def forward(self, h, meta, cache: LayerCache):
+        s = self.s
+        H, D, Dv = s.heads, s.dim, s.vdim
+        qkvg = ops.linear(h, self.qkvg.data)
+        # rotation, key scale and everything behind them in fp32, whatever the model dtype
+        qkv = seqmix.retention_prep(qkvg, meta.positions, self.inv_freq, s.rot_dims, H, D, Dv, D ** -0.5)
+        o = seqmix.lightning_scan(qkv, cache.state, meta, H, D, Dv, self.decay, activation="none")
+        y = seqmix.rms_gate(o, None, self.eps, qkvg[:, 2 * H * D + H * Dv:], h.dtype, groups=H, gate_act="silu")
+        return ops.linear(y, self.o.data)
+
+
+MIXERS = {"gated_attention": GatedAttention, "retention": Retention, "attention": WindowAttention, "latent_attention": LatentAttention, "lightning": LightningAttention,
           "sink_attention": SinkTalkAttention, "time_mix": TimeMix, "parallel": DualMixer}
 
 
@@ -341,6 +428,128 @@ class RoutedFF(nn.Module):
             if s.shared_ff:
                 shared = ops.linear(seqmix.relu2_rows(both[:, :s.shared_ff]), self.shared_down.data)
         return routed, shared, sgate, extra
+
+
+class GatedDenseFF(nn.Module):
+    """``W_down · (act(W_gate h) ⊙ W_up h)``; gate and up rows are one GEMM."""
+
+    def __init__(self, width: int, ff: int, act: str, ctx, dtype, device):
+        super().__init__()
+        self.act = act
+        self.gate_up, self.down = _matrix(2 * ff, width, ctx, dtype, device), _matrix(width, ff, ctx, dtype, device)
+
+    def weights(self, p):
+        yield p + "gate_up", self.gate_up, "normal", [p + "gate", p + "up"]
+        yield p + "down", self.down, "normal", None
+
+    def forward(self, h):
+        return ops.linear(seqmix.act_mul(ops.linear(h, self.gate_up.data), self.act), self.down.data)
+
+
+class SoftmaxRoutedFF(nn.Module):
+    """``Σ_chosen p_e · expert_e(h)``, ``expert(h) = W_down · (silu(W_gate h) ⊙ W_up h)``: the ``top`` experts with the largest
+    fp32 router logits ``W_r h + b`` are chosen, ``p`` is the softmax over the chosen logits."""
+
+    def __init__(self, spec: MixerSpec, width: int, ctx, dtype, device):
+        super().__init__()
+        self.s = spec
+        E, F = spec.experts, spec.ff
+        assert 1 <= spec.top <= E
+        if spec.ff_act != "silu":
+            raise ValueError(f"routed gated experts use silu, not {spec.ff_act!r}")
+        self.gate_up, self.down = Weight((E, 2 * F, width), None, ctx, dtype, device), Weight((E, width, F), None, ctx, dtype, device)
+        self.router, self.bias = _param((E, width), ctx, device), _param((E,), ctx, device)
+
+    def weights(self, p):
+        E = self.s.experts
+        yield p + "experts.gate_up", self.gate_up, "normal", [[p + f"e{e}.gate", p + f"e{e}.up"] for e in range(E)]
+        yield p + "experts.down", self.down, "normal", [[p + f"e{e}.down"] for e in range(E)]
+        yield p + "router", self.router, "normal", None
+        yield p + "router.b", self.bias, "zeros", None
+
+    def forward(self, h):
+        ids, wts = seqmix.softmax_route(h, self.router.data, self.bias.data, self.s.top)
+        return seqmix.gated_experts(h, ids, wts, self.gate_up.data, self.down.data)
+
+
+class StreamLinks(nn.Module):
+    """How one sublayer reads and writes ``S`` copies of the stream: ``u = Σ_s in[s] x_s`` goes in; the result ``y`` comes back
+    as ``x_t ← Σ_s mix[s, t] x_s + out[t] y``.  ``S = 1`` with all-ones weights is the plain residual sum."""
+
+    def __init__(self, streams: int, ctx, device):
+        super().__init__()
+        self.w_in, self.w_out, self.mix = _param((streams,), ctx, device), _param((streams,), ctx, device), _param((streams, streams), ctx, device)
+        with torch.no_grad():           # the plain residual sum until a checkpoint or the random initialisation says otherwise
+            self.w_in.init_const(1.0)
+            self.w_out.init_const(1.0)
+            self.mix.load_full(torch.eye(streams, dtype=torch.float32, device=device))
+
+    def weights(self, p):
+        yield p + "in", self.w_in, "ones", None
+        yield p + "out", self.w_out, "ones", None
+        yield p + "mix", self.mix, "eye", None
+
+
+class HyperLayer(nn.Module):
+    """Pre-norm layer over ``S`` fp32 streams ``x [T, S, W]``: ``y = mixer(conv(norm1(Σ in·x)))`` written back through the first
+    links, then ``y = ff(norm2(Σ in·x))`` through the second.  Norm weights are stored around zero (``1 + w``); ``conv`` adds a
+    causal per-channel convolution over the sequence's last ``taps`` inputs (``taps`` = 0: none).  ``links`` False: one stream,
+    plain residual sums (the link weights stay at one and are not part of a checkpoint)."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, streams: int, taps: int, ctx: ParallelContext, dtype, device):
+        super().__init__()
+        self.spec, self.eps, self.dtype, self.taps = spec, eps, dtype, taps
+        self.links = streams > 0
+        S = max(streams, 1)
+        self.norm1, self.hc1 = _param((width,), ctx, device), StreamLinks(S, ctx, device)
+        self.conv = _param((width, taps), ctx, device) if taps else None
+        self.mixer = MIXERS[spec.kind](spec, width, eps, ctx, dtype, device)
+        self.ff = None
+        if spec.ff:
+            self.norm2, self.hc2 = _param((width,), ctx, device), StreamLinks(S, ctx, device)
+            if spec.ff_kind == "moe":
+                if spec.router != "softmax":
+                    raise ValueError(f"hyper-connected layers route by softmax, not {spec.router!r}")
+                self.ff = SoftmaxRoutedFF(spec, width, ctx, dtype, device)
+            else:
+                self.ff = GatedDenseFF(width, spec.ff, spec.ff_act, ctx, dtype, device)
+
+    def weights(self, p):
+        yield p + "norm1", self.norm1, "zeros", None
+        if self.links:
+            yield from self.hc1.weights(p + "hc1.")
+        if self.conv is not None:
+            yield p + "canon1", self.conv, "small", None
+        yield from self.mixer.weights(p + "mix.")
+        if self.ff is not None:
+            yield p + "norm2", self.norm2, "zeros", None
+            if self.links:
+                yield from self.hc2.weights(p + "hc2.")
+            yield from self.ff.weights(p + "mlp.")
+
+    def cache(self, num_blocks, num_slots, dtype, device) -> LayerCache:
+        c = self.mixer.cache(num_blocks, num_slots, dtype, device)
+        if self.taps > 1:           # the sequence's last taps-1 mixer inputs, oldest first
+            c.shift = torch.zeros(num_slots, self.taps - 1, self.norm1.data.shape[0], dtype=torch.float32, device=device)
+        return c
+
+    def read(self, x, y, prev: Optional[StreamLinks], out_dtype):
+        """Write the previous sublayer's ``y`` back through its links ``prev`` (if any) and return this layer's mixer input
+        before the convolution."""
+        return seqmix.stream_mix_norm(x, y, prev.mix.data if prev else None, prev.w_out.data if prev else None, self.hc1.w_in.data,
+                                      self.norm1.data, self.eps, 1.0, out_dtype)
+
+    def forward(self, x, h, meta, cache: LayerCache):
+        """``x``: fp32 streams ``[T, S, W]``, updated in place; ``h``: this layer's normed mixer input (``read``).  Returns the
+        last sublayer's output and its links — the caller's next ``read`` (or the closing norm) writes them back."""
+        if self.conv is not None:
+            h = seqmix.causal_conv_add(h, self.conv.data, cache.shift, meta, self.dtype)
+        y = self.mixer(h, meta, cache)
+        if self.ff is None:
+            return y, self.hc1
+        h2 = seqmix.stream_mix_norm(x, y, self.hc1.mix.data, self.hc1.w_out.data, self.hc2.w_in.data, self.norm2.data, self.eps, 1.0,
+                                    self.dtype)
+        return self.ff(h2), self.hc2
 
 
 class GatedParallelLayer(nn.Module):

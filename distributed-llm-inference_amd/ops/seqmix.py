@@ -100,13 +100,23 @@ def add_ln(x: torch.Tensor, y: torch.Tensor, w: torch.Tensor, b: torch.Tensor, e
     return None if w2 is None else _ln(x, w2, b2, eps).to(out_dtype)
 
 
-def rms_gate(o: torch.Tensor, w: torch.Tensor, eps: float, gate: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """``o / rms(o) · w · sigmoid(gate)`` per row (``o`` fp32 ``[T, N]``, or — what the GPU scan returns — planes of partial
-    sums ``[parts, T, N]`` whose sum is the row; ``gate`` a row-strided view)."""
+def rms_gate(o: torch.Tensor, w: Optional[torch.Tensor], eps: float, gate: torch.Tensor, out_dtype: torch.dtype, groups: int = 1,
+             gate_act: str = "sigmoid") -> torch.Tensor:
+    """``o / rms(o) · w · act(gate)`` per row (``o`` fp32 ``[T, N]``, or — what the GPU scan returns — planes of partial
+    sums ``[parts, T, N]`` whose sum is the row; ``gate`` a row-strided view).  ``groups`` > 1: every one of that many equal
+    slices of the row is divided by its own root mean square; ``w`` None: no weight; ``gate_act``: ``"sigmoid"`` or ``"silu"``."""
+    assert gate_act in ("sigmoid", "silu")
     if o.is_cuda:
-        return _hip().sm_rms_gate(o, w, eps, gate, out_dtype == torch.bfloat16)
-    y = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps) * w
-    return (y * torch.sigmoid(gate.float())).to(out_dtype)
+        return _hip().sm_rms_gate(o, w, eps, gate, out_dtype == torch.bfloat16, groups, gate_act == "silu")
+    if o.dim() == 3:
+        o = o.sum(0)
+    T, N = o.shape
+    g = o.view(T, groups, N // groups)
+    y = (g * torch.rsqrt((g * g).mean(-1, keepdim=True) + eps)).reshape(T, N)
+    if w is not None:
+        y = y * w
+    z = gate.float()
+    return (y * (torch.sigmoid(z) if gate_act == "sigmoid" else torch.nn.functional.silu(z))).to(out_dtype)
 
 
 def relu2(x: torch.Tensor) -> torch.Tensor:
@@ -182,13 +192,14 @@ def latent_prep(q: torch.Tensor, dkv: torch.Tensor, cw: torch.Tensor, eps: float
 def token_attention(out: torch.Tensor, q1: torch.Tensor, q2: Optional[torch.Tensor], k_cache: torch.Tensor,
                     v_cache: Optional[torch.Tensor], meta, G: int, Dv: int, scale: float, window: int = 0,
                     temp: Optional[torch.Tensor] = None, r1: Optional[torch.Tensor] = None,
-                    r2: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    r2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Softmax attention of this step's tokens over their sequences' cached rows (which already hold this step's keys).
 
     ``q1 [T, H, D1]`` (and ``q2 [T, H, D2]``) against key rows ``[G, D1 + D2]``: ``score = (q1·k[:D1] + q2·k[D1:]) · scale ·
     temp[h] − r1[h] · ln(1 + r2[h] · distance)``; query head ``h`` reads key / value head ``h // (H/G)``.  ``v_cache`` None:
     the values are the first ``Dv`` entries of the key rows (latent attention: the cached latent is key and value).
-    ``window`` > 0: a query at position ``p`` sees positions ``p-window+1 … p``; 0: all up to ``p``.  Views may be strided
+    ``window`` > 0: a query at position ``p`` sees positions ``p-window+1 … p``; 0: all up to ``p``.  ``gate [T, H]``
+    (pre-activation, row-strided view): head ``h``'s result is multiplied by ``sigmoid(gate[t, h])``.  Views may be strided
     (last dim contiguous).  Writes ``out [T, H, Dv]``."""
     if _act_ok(q1):
         lib = _hip()
@@ -197,17 +208,17 @@ def token_attention(out: torch.Tensor, q1: torch.Tensor, q2: Optional[torch.Tens
             # prefill chunks: 64-query tiles on the matrix cores; the per-token kernel keeps the decode rows in front
             if lib.sm_tile_attention(out, q1, q2, k_cache, v_cache, meta.block_tables, meta.seq_lens, meta.query_start_loc,
                                      meta.prefill_tile_seq, meta.prefill_tile_q0, meta.num_prefill_tiles,
-                                     meta.counts if meta.counts_on_device else None, G, Dv, scale, window, temp, r1, r2):
+                                     meta.counts if meta.counts_on_device else None, G, Dv, scale, window, temp, r1, r2, gate):
                 rows = meta.num_decode
         T, H = q1.shape[0], q1.shape[1]
         todo = T if rows < 0 else rows                       # tokens the tile kernel left (all of them in a pure decode step)
         if (HEAD_DECODE and todo > 0 and q1.dtype == torch.bfloat16 and H // G >= 8 and meta.num_prefill_tiles == (0 if rows < 0 else meta.num_prefill_tiles)
                 and lib.sm_head_decode_attention(out, q1, q2, k_cache, v_cache, meta.block_tables, meta.positions, meta.token_seq,
-                                                 G, Dv, scale, window, temp, r1, r2, todo)):
+                                                 G, Dv, scale, window, temp, r1, r2, todo, gate)):
             rows = 0                                         # done with the heads as matrix-core columns
         if rows != 0:
             lib.sm_token_attention(out, q1, q2, k_cache, v_cache, meta.block_tables, meta.positions, meta.token_seq,
-                                   G, Dv, scale, window, temp, r1, r2, rows)
+                                   G, Dv, scale, window, temp, r1, r2, rows, gate)
         return out
     T, H, D1 = q1.shape
     rowk = k_cache.shape[-1]
@@ -242,24 +253,32 @@ def token_attention(out: torch.Tensor, q1: torch.Tensor, q2: Optional[torch.Tens
         if window > 0:
             hidden = hidden | (dist >= window)
         s = s.masked_fill(hidden.unsqueeze(1), float("-inf"))
-        out[t0:t1] = torch.einsum("nhl,lhd->nhd", torch.softmax(s, dim=-1), Vh).to(out.dtype)
+        o = torch.einsum("nhl,lhd->nhd", torch.softmax(s, dim=-1), Vh)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[t0:t1].float()).unsqueeze(2)
+        out[t0:t1] = o.to(out.dtype)
     return out
 
 
 # ------------------------------------------------------------------------------------ decayed linear attention
-def lightning_scan(qkvg: torch.Tensor, state: torch.Tensor, meta, H: int, D: int, Dv: int, decay: torch.Tensor) -> torch.Tensor:
-    """``qkvg [T, 2·H·D + 2·H·Dv]`` = ``[q | k | v | gate]`` (pre-activation; the gate columns are not read).  Per sequence
-    and head, token by token: ``S ← decay[h] · S + silu(k) silu(v)ᵀ``, ``o = Sᵀ silu(q)`` with ``S`` = the sequence's fp32
-    ``state[slot, h]`` ``[D, Dv]`` (zero at position 0), written back after the step's last token.  Returns fp32 ``[T, H·Dv]`` (GPU: ``[parts, T, H·Dv]``
-    partial sums over parts of the state rows, for ``rms_gate``)."""
+def lightning_scan(qkvg: torch.Tensor, state: torch.Tensor, meta, H: int, D: int, Dv: int, decay: torch.Tensor,
+                   activation: str = "silu") -> torch.Tensor:
+    """``qkvg [T, 2·H·D + 2·H·Dv]`` = ``[q | k | v | gate]`` (pre-activation; the gate columns are not read and may be
+    missing).  Per sequence and head, token by token: ``S ← decay[h] · S + act(k) act(v)ᵀ``, ``o = Sᵀ act(q)`` with ``S`` = the
+    sequence's fp32 ``state[slot, h]`` ``[D, Dv]`` (zero at position 0), written back after the step's last token; ``act`` is
+    silu, or the identity with ``activation="none"``.  Returns fp32 ``[T, H·Dv]`` (GPU: ``[parts, T, H·Dv]`` partial sums over
+    parts of the state rows, for ``rms_gate``)."""
+    assert activation in ("silu", "none")
     if _act_ok(qkvg):
         # prefill chunks run block-parallel over the step's 64-token tiles (local states → prefix over blocks → outputs)
         tiles = meta.num_prefill_tiles if BLOCK_SCAN else 0
         return _hip().sm_lightning_scan(qkvg, state, meta.positions, meta.query_start_loc, meta.state_slots, meta.counts,
                                         meta.num_seqs, H, D, Dv, decay, meta.prefill_tile_seq if tiles else None,
-                                        meta.prefill_tile_q0 if tiles else None, tiles)
+                                        meta.prefill_tile_q0 if tiles else None, tiles, activation == "none")
     T = qkvg.shape[0]
-    act = torch.nn.functional.silu(qkvg[:, :2 * H * D + H * Dv].float())
+    act = qkvg[:, :2 * H * D + H * Dv].float()
+    if activation == "silu":
+        act = torch.nn.functional.silu(act)
     q, k, v = act[:, :H * D].view(T, H, D), act[:, H * D:2 * H * D].view(T, H, D), act[:, 2 * H * D:].view(T, H, Dv)
     o = torch.zeros(T, H, Dv)
     B = meta.num_decode + meta.num_prefill
@@ -336,19 +355,23 @@ def stretched_inv_freq(base: float, dims: int, scaling: tuple = (), device="cpu"
 
 
 def wide_norm_rope_cache(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor, eps: float, positions: torch.Tensor,
-                         inv_freq: torch.Tensor, mag: float, rot_dims: int, slot_mapping: torch.Tensor, k_cache: torch.Tensor,
-                         v_cache: torch.Tensor, H: int, G: int, D: int, Dv: int) -> None:
+                         inv_freq: Optional[torch.Tensor], mag: float, rot_dims: int, slot_mapping: torch.Tensor,
+                         k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], H: int, G: int, D: int, Dv: int) -> None:
     """Leading columns of ``qkv`` rows = ``[q (H·D) | k (G·D) | v (G·Dv)]``.  The whole q row and the whole k row are each
     divided by their root mean square (over all heads at once) and multiplied by ``qw`` / ``kw``; then entries ``i`` and
     ``i + rot_dims/2`` (``i < rot_dims/2``) of every head are turned by ``position · inv_freq[i]`` with cosine and sine
-    scaled by ``mag``.  q is written back in place; k and v go to the token-major cache rows ``slot_mapping`` (< 0: skipped)."""
+    scaled by ``mag``.  q is written back in place; k and v go to the token-major cache rows ``slot_mapping`` (< 0: skipped).
+    ``G = 0`` (no caches, ``kw`` unused): the rows hold queries only — a mixer that reads another layer's keys and values.
+    ``inv_freq`` may be None when nothing is rotated."""
     if _act_ok(qkv):
-        _hip().dm_wide_norm_rope_cache(qkv, qw, kw, eps, positions, inv_freq, mag, rot_dims, slot_mapping, k_cache, v_cache, H, G, D, Dv)
+        _hip().dm_wide_norm_rope_cache(qkv, qw, kw if G else None, eps, positions, inv_freq if rot_dims else None, mag, rot_dims,
+                                       slot_mapping, k_cache if G else None, v_cache if G else None, H, G, D, Dv)
         return
     T = qkv.shape[0]
     q, k = qkv[:, :H * D].float(), qkv[:, H * D:(H + G) * D].float()
     q = (q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * qw).view(T, H, D)
-    k = (k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * kw).view(T, G, D)
+    if G:
+        k = (k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * kw).view(T, G, D)
     if rot_dims:
         ang = positions.double()[:, None] * inv_freq[None, :]
         cos, sin = (ang.cos() * mag).float().unsqueeze(1), (ang.sin() * mag).float().unsqueeze(1)
@@ -357,8 +380,11 @@ def wide_norm_rope_cache(qkv: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor, 
         def turn(v):
             a, b = v[..., :half], v[..., half:rot_dims]
             return torch.cat([a * cos - b * sin, b * cos + a * sin, v[..., rot_dims:]], dim=-1)
-        q, k = turn(q), turn(k)
+        q = turn(q)
+        k = turn(k) if G else k
     qkv[:, :H * D] = q.reshape(T, H * D).to(qkv.dtype)
+    if not G:
+        return
     keep = slot_mapping >= 0
     s = slot_mapping[keep].long()
     k_cache.view(-1, G * D)[s] = k.reshape(T, G * D)[keep].to(k_cache.dtype)
@@ -465,7 +491,7 @@ def sigmoid_route(h: torch.Tensor, router: torch.Tensor, experts: int, top: int,
 def relu2_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
     """``Σ_slots wts[t, s] · down[e] · relu(up[e] · h[t])²`` with ``e = ids[t, s]``; ``up [E, F, W]``, ``down [E, W, F]``."""
     if _act_ok(h):
-        return _hip().dm_relu2_experts(h, ids, wts, up, down)
+        return _hip().dm_relu2_experts(h, ids, wts, up, down, False)
     out = torch.zeros(h.shape[0], h.shape[1])
     hf = h.float()
     for e in range(up.shape[0]):
@@ -501,3 +527,114 @@ def gated_combine(x: torch.Tensor, mult: float, parts: list, scales: list, gate1
             f = f + shared.float() * (shared_gate.unsqueeze(1) if shared_gate is not None else 1.0)
         y = y + f * torch.sigmoid(gate2.float() + b2)
     x.add_(y, alpha=mult)
+
+
+# ====================================================================================== hyper-connected stacks
+# Ops of stacks that keep several copies of the residual stream, add a short causal convolution to every mixer's input and
+# mix gated attention / retention layers with gated dense or softmax-routed feed-forwards (``models/mixers.py``:
+# ``GatedAttention``, ``Retention``, ``GatedDenseFF``, ``SoftmaxRoutedFF``, ``HyperLayer``).  GPU kernels:
+# ``csrc/kernels/hypermix.hip`` (``torch.ops.dli.hm_*``) beside extensions of the kernels above.
+def stream_mix_norm(x: torch.Tensor, y: Optional[torch.Tensor], mix: Optional[torch.Tensor], out_w: Optional[torch.Tensor],
+                    in_w: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], eps: float, w_offset: float,
+                    out_dtype: torch.dtype) -> Optional[torch.Tensor]:
+    """One pass over the fp32 streams ``x [T, S, W]``.  With ``y [T, W]`` (a sublayer's output): all streams at once from the
+    old ones, in place, ``x[:, t] ← Σ_s mix[s, t] · x[:, s] + out_w[t] · y``.  With ``in_w [S]``: returns
+    ``rms_norm(Σ_s in_w[s] · x[:, s]) · (w_offset + norm_w)`` in ``out_dtype`` — what the next sublayer (or the LM head)
+    reads, computed from the updated streams."""
+    if x.is_cuda:
+        h = _hip().hm_stream_mix_norm(x, y, mix, out_w, in_w, norm_w, eps, w_offset, out_dtype == torch.bfloat16)
+        return h if in_w is not None else None
+    if y is not None:
+        new = torch.einsum("st,nsw->ntw", mix, x) + out_w.view(1, -1, 1) * y.float().unsqueeze(1)
+        x.copy_(new)
+    if in_w is None:
+        return None
+    u = torch.einsum("s,nsw->nw", in_w, x)
+    return (u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps) * (w_offset + norm_w)).to(out_dtype)
+
+
+def causal_conv_add(h: torch.Tensor, w: torch.Tensor, state: torch.Tensor, meta, out_dtype: torch.dtype) -> torch.Tensor:
+    """``h [T, W]`` fp32; ``w [W, taps]`` fp32.  Row ``t`` of the result is ``h[t] + Σ_j w[:, j] · h[t - taps + 1 + j]`` over the
+    rows of the same sequence: rows above inside a chunk, the sequence's ``state`` rows ``[slots, taps-1, W]`` (its last
+    ``taps-1`` inputs, oldest first) before a chunk's start, zero before position 0.  The state rows are then moved on to
+    the sequence's last ``taps-1`` inputs of this step."""
+    if h.is_cuda:
+        return _hip().hm_causal_conv_add(h, w, state, meta.positions, meta.token_seq, meta.query_start_loc, meta.state_slots,
+                                         meta.counts, meta.num_seqs, out_dtype == torch.bfloat16)
+    taps = w.shape[1]
+    out = h.clone()
+    for _i, t0, t1, slot in _seq_rows(meta):
+        p0 = int(meta.positions[t0])
+        n = t1 - t0
+        hist = state[slot].clone() if taps > 1 else h.new_zeros(0, h.shape[1])          # positions p0-(taps-1) … p0-1
+        for r in range(taps - 1):
+            if p0 - (taps - 1) + r < 0:
+                hist[r] = 0.0
+        ext = torch.cat([hist, h[t0:t1]], dim=0)                                         # [taps-1+n, W]
+        for j in range(taps):
+            out[t0:t1] += w[:, j] * ext[j:j + n]
+        if taps > 1:
+            state[slot] = ext[n:]
+    return out.to(out_dtype)
+
+
+def retention_prep(qkvg: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rot_dims: int, H: int, D: int,
+                   Dv: int, k_scale: float) -> torch.Tensor:
+    """fp32 ``[T, 2·H·D + H·Dv]`` = ``[q' | k' | v]`` from the leading columns ``[q | k | v]`` of ``qkvg``: in every head of q
+    and k, entries ``i`` and ``i + rot_dims/2`` (``i < rot_dims/2``) are turned by ``position · inv_freq[i]``; k is then
+    multiplied by ``k_scale``."""
+    if _act_ok(qkvg):
+        return _hip().hm_retention_prep(qkvg, positions, inv_freq if rot_dims else None, rot_dims, H, D, Dv, k_scale)
+    T = qkvg.shape[0]
+    x = qkvg[:, :2 * H * D + H * Dv].float().clone()
+    qk = x[:, :2 * H * D].view(T, 2 * H, D)
+    if rot_dims:
+        ang = positions.double()[:T, None] * inv_freq[None, :]
+        cos, sin = ang.cos().float().unsqueeze(1), ang.sin().float().unsqueeze(1)
+        half = rot_dims // 2
+        a, b = qk[..., :half].clone(), qk[..., half:rot_dims].clone()
+        qk[..., :half] = a * cos - b * sin
+        qk[..., half:rot_dims] = b * cos + a * sin
+    qk[:, H:] *= k_scale
+    return x
+
+
+def act_mul(x: torch.Tensor, kind: str) -> torch.Tensor:
+    """``act(x[:, :F]) · x[:, F:]`` of rows ``[T, 2F]``; ``kind``: ``"gelu_tanh"`` (``0.5 z (1 + tanh(√(2/π) (z + 0.044715 z³)))``)
+    or ``"silu"``."""
+    assert kind in ("gelu_tanh", "silu")
+    if _act_ok(x):
+        return _hip().hm_act_mul(x, kind == "silu")
+    F = x.shape[1] // 2
+    a, b = x[:, :F].float(), x[:, F:].float()
+    a = torch.nn.functional.gelu(a, approximate="tanh") if kind == "gelu_tanh" else torch.nn.functional.silu(a)
+    return (a * b).to(x.dtype)
+
+
+def softmax_route(h: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+    """fp32 logits ``router · h + bias`` per token (``router`` fp32 ``[E, W]``); the ``top`` experts with the largest logits
+    (ties: lowest index) and the softmax over the chosen logits only.  Returns ``(ids int32 [T, top], weights fp32 [T, top])``."""
+    if _act_ok(h):
+        return _hip().hm_softmax_route(h, router, bias, top)
+    z = h.float() @ router.t()
+    if bias is not None:
+        z = z + bias
+    val, ids = torch.sort(z, dim=-1, descending=True, stable=True)
+    return ids[:, :top].int(), torch.softmax(val[:, :top], dim=-1)
+
+
+def gated_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
+    """``Σ_slots wts[t, s] · down[e] · (silu(gate[e] · h[t]) ⊙ up[e] · h[t])`` with ``e = ids[t, s]``; ``gate_up [E, 2F, W]``
+    (an expert's gate rows, then its up rows), ``down [E, W, F]``."""
+    if _act_ok(h):
+        return _hip().dm_relu2_experts(h, ids, wts, gate_up, down, True)
+    F = gate_up.shape[1] // 2
+    out = torch.zeros(h.shape[0], h.shape[1])
+    hf = h.float()
+    for e in range(gate_up.shape[0]):
+        tok, slot = torch.nonzero(ids == e, as_tuple=True)
+        if tok.numel():
+            gu = hf[tok] @ gate_up[e].float().t()
+            a = (torch.nn.functional.silu(gu[:, :F]) * gu[:, F:]).to(h.dtype).float()
+            out.index_add_(0, tok, (a @ down[e].float().t()) * wts[tok, slot].unsqueeze(1))
+    return out.to(h.dtype)
