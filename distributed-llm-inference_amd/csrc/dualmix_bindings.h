@@ -47,33 +47,46 @@ Tensor dm_shift_mix(const Tensor& h, const Tensor& mu, Tensor state, const Tenso
   return out;
 }
 
-void dm_wide_norm_rope_cache(Tensor qkv, const Tensor& qw, const Tensor& kw, double eps, const Tensor& positions, const Tensor& freq,
-                             double mag, int64_t rot_dims, const Tensor& slot_mapping, Tensor k_cache, Tensor v_cache, int64_t H,
-                             int64_t G, int64_t D, int64_t Dv) {
+// G = 0: the rows hold queries only (kw and both caches absent); rot_dims = 0: nothing is rotated (freq may be absent)
+void dm_wide_norm_rope_cache(Tensor qkv, const Tensor& qw, const c10::optional<Tensor>& kw, double eps, const Tensor& positions,
+                             const c10::optional<Tensor>& freq, double mag, int64_t rot_dims, const Tensor& slot_mapping,
+                             const c10::optional<Tensor>& k_cache, const c10::optional<Tensor>& v_cache, int64_t H, int64_t G, int64_t D,
+                             int64_t Dv) {
   const bool bf = act_bf16(qkv, "qkv");
   check_rows(qkv, "qkv");
   const int64_t T = qkv.size(0);
-  TORCH_CHECK(H > 0 && G > 0 && D > 0 && Dv > 0 && qkv.size(1) >= H * D + G * D + G * Dv, "qkv rows shorter than q | k | v");
+  TORCH_CHECK(H > 0 && G >= 0 && D > 0 && Dv > 0 && qkv.size(1) >= H * D + G * D + G * Dv, "qkv rows shorter than q | k | v");
   check_f32(qw, "qw", H * D);
-  check_f32(kw, "kw", G * D);
+  TORCH_CHECK((G > 0) == kw.has_value() && (G > 0) == k_cache.has_value() && (G > 0) == v_cache.has_value(),
+              "key weights and both caches come with key / value heads, and only with them");
+  const float* kwp = opt_f32(kw, "kw", G * D);
   TORCH_CHECK(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= D, "rot_dims must be even and at most D");
   TORCH_CHECK(rot_dims / 2 <= 256, "too many rotated pairs");
-  TORCH_CHECK(freq.is_cuda() && freq.scalar_type() == at::kDouble && freq.is_contiguous() && freq.numel() >= rot_dims / 2,
-              "freq must be a float64 GPU tensor [rot_dims / 2]");
+  const double* fp = nullptr;
+  if (rot_dims > 0) {
+    TORCH_CHECK(freq.has_value() && freq->is_cuda() && freq->scalar_type() == at::kDouble && freq->is_contiguous() &&
+                    freq->numel() >= rot_dims / 2, "freq must be a float64 GPU tensor [rot_dims / 2]");
+    fp = freq->data_ptr<double>();
+  }
   check_i32(positions, "positions");
   check_i32(slot_mapping, "slot_mapping");
   TORCH_CHECK(positions.numel() >= T && slot_mapping.numel() >= T, "step metadata shorter than the batch");
-  check_act_like(k_cache, bf, "k_cache");
-  check_act_like(v_cache, bf, "v_cache");
-  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous() && k_cache.dim() == 3 && v_cache.dim() == 3 &&
-                  k_cache.size(1) == kSmPageTokens && v_cache.size(1) == kSmPageTokens && k_cache.size(2) == G * D &&
-                  v_cache.size(2) == G * Dv && k_cache.size(0) == v_cache.size(0),
-              "caches must be [pages, 32, G*D] and [pages, 32, G*Dv]");
+  void* kp = nullptr;
+  void* vp = nullptr;
+  if (G > 0) {
+    check_act_like(*k_cache, bf, "k_cache");
+    check_act_like(*v_cache, bf, "v_cache");
+    TORCH_CHECK(k_cache->is_contiguous() && v_cache->is_contiguous() && k_cache->dim() == 3 && v_cache->dim() == 3 &&
+                    k_cache->size(1) == kSmPageTokens && v_cache->size(1) == kSmPageTokens && k_cache->size(2) == G * D &&
+                    v_cache->size(2) == G * Dv && k_cache->size(0) == v_cache->size(0),
+                "caches must be [pages, 32, G*D] and [pages, 32, G*Dv]");
+    kp = k_cache->data_ptr();
+    vp = v_cache->data_ptr();
+  }
   TORCH_CHECK((H * D + G * D + rot_dims) * 4 <= kSmMaxLds, "q and k rows too wide");
-  dli::launch_dm_wide_norm_rope_cache(qkv.data_ptr(), bf, qkv.stride(0), qw.data_ptr<float>(), kw.data_ptr<float>(), (float)eps,
-                                      positions.data_ptr<int>(), freq.data_ptr<double>(), (float)mag, (int)rot_dims,
-                                      slot_mapping.data_ptr<int>(), k_cache.data_ptr(), v_cache.data_ptr(), (int)T, (int)H, (int)G, (int)D,
-                                      (int)Dv, cur_stream(qkv));
+  dli::launch_dm_wide_norm_rope_cache(qkv.data_ptr(), bf, qkv.stride(0), qw.data_ptr<float>(), kwp, (float)eps,
+                                      positions.data_ptr<int>(), fp, (float)mag, (int)rot_dims, slot_mapping.data_ptr<int>(), kp, vp,
+                                      (int)T, (int)H, (int)G, (int)D, (int)Dv, cur_stream(qkv));
 }
 
 void dm_talk_attention(Tensor out, const Tensor& q, const c10::optional<Tensor>& gate, const Tensor& k_cache, const Tensor& v_cache,
@@ -231,21 +244,29 @@ std::tuple<Tensor, Tensor, Tensor> dm_sigmoid_route(const Tensor& h, const Tenso
 bool g_dm_grouped_experts = true;     // A/B knob (dm_set_grouped_experts): routed experts as grouped GEMMs on the matrix cores
 void dm_set_grouped_experts(bool on) { g_dm_grouped_experts = on; }
 
-Tensor dm_relu2_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, const Tensor& up, const Tensor& down) {
+// gated: `up` holds an expert's gate rows, then its up rows ([E, 2F, W]); the activation is silu(gate · h) ⊙ (up · h)
+Tensor dm_relu2_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, const Tensor& up, const Tensor& down, bool gated) {
   const bool bf = act_bf16(h, "h");
   check_rows(h, "h");
   const int64_t T = h.size(0), W = h.size(1);
   check_act_like(up, bf, "up");
   check_act_like(down, bf, "down");
   TORCH_CHECK(up.dim() == 3 && down.dim() == 3 && up.is_contiguous() && down.is_contiguous(), "expert weights must be contiguous 3-D");
-  const int64_t E = up.size(0), F = up.size(1);
-  TORCH_CHECK(up.size(2) == W && down.size(0) == E && down.size(1) == W && down.size(2) == F, "expert weights must be [E, F, W] and [E, W, F]");
+  const int64_t E = up.size(0), F = gated ? up.size(1) / 2 : up.size(1);
+  TORCH_CHECK(up.size(1) == (gated ? 2 * F : F) && up.size(2) == W && down.size(0) == E && down.size(1) == W && down.size(2) == F,
+              "expert weights must be [E, F (gated: 2F), W] and [E, W, F]");
   check_i32(ids, "ids");
   check_f32(wts, "wts");
   TORCH_CHECK(ids.dim() == 2 && ids.size(0) == T && wts.dim() == 2 && wts.size(0) == T && wts.size(1) == ids.size(1), "ids / wts must be [T, K]");
   const int64_t K = ids.size(1);
   Tensor out = at::empty({T, W}, h.options());
-  if (bf && g_dm_grouped_experts && W % 128 == 0 && F % 128 == 0 && E <= 64 && T * K >= 64 && h.stride(0) % 8 == 0 &&
+  if (gated && bf && g_dm_grouped_experts && W % 128 == 0 && F % 64 == 0 && E <= 64 && T * K >= 64 && h.is_contiguous() &&
+      reinterpret_cast<uintptr_t>(h.data_ptr()) % 16 == 0) {
+    // the grouped GEMMs of the Mixtral path (gate / up tile pairs with the silu product in the first epilogue)
+    moe_experts_forward(h, ids, wts, up, down, K, 0, false, out.data_ptr(), cur_stream(h));
+    return out;
+  }
+  if (!gated && bf && g_dm_grouped_experts && W % 128 == 0 && F % 128 == 0 && E <= 64 && T * K >= 64 && h.stride(0) % 8 == 0 &&
       reinterpret_cast<uintptr_t>(h.data_ptr()) % 16 == 0) {
     // matrix-core path: the routed rows are bucketed by expert and both projections run as grouped GEMMs on 128-row tiles
     // (kernels/moe.hip: rows gathered by index, relu² in the first epilogue, gate weight and scatter in the second)
@@ -276,7 +297,7 @@ Tensor dm_relu2_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, c
   TORCH_CHECK(W * 4 <= kSmMaxLds && K * F * 4 <= kSmMaxLds, "rows too wide");
   Tensor act = at::empty({T * K, F}, h.options());
   dli::launch_dm_experts(h.data_ptr(), bf, h.stride(0), ids.data_ptr<int>(), wts.data_ptr<float>(), (int)K, up.data_ptr(), down.data_ptr(),
-                         (int)T, (int)F, (int)W, act.data_ptr(), out.data_ptr(), cur_stream(h));
+                         (int)T, (int)F, (int)W, act.data_ptr(), out.data_ptr(), gated, cur_stream(h));
   return out;
 }
 

@@ -149,7 +149,7 @@ __global__ __launch_bounds__(NT) void wide_norm_rope_cache_kernel(A* __restrict_
     ks[i] = v;
     sk += v * v;
   }
-  if (threadIdx.x < half) {
+  if (threadIdx.x < half && freq != nullptr) {
     const double two_pi = 6.283185307179586476925286766559;
     double a = (double)positions[t] * freq[threadIdx.x];
     a -= floor(a / two_pi) * two_pi;
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(NT) void wide_norm_rope_cache_kernel(A* __restrict_
     sn[threadIdx.x] = sinf((float)a) * mag;
   }
   const float iq = 1.f / sqrtf(block_sum<NT>(sq, red) / (float)nq + eps);
-  const float ik = 1.f / sqrtf(block_sum<NT>(sk, red) / (float)nk + eps);
+  const float ik = 1.f / sqrtf(block_sum<NT>(sk, red) / (float)max(nk, 1) + eps);        // nk = 0: queries only
   for (int i = threadIdx.x; i < nq; i += NT) qs[i] = qs[i] * iq * qw[i];
   for (int i = threadIdx.x; i < nk; i += NT) ks[i] = ks[i] * ik * kw[i];
   __syncthreads();
@@ -172,7 +172,7 @@ __global__ __launch_bounds__(NT) void wide_norm_rope_cache_kernel(A* __restrict_
     if (i < nq) stf<A>(row + i, v);
     else if (slot >= 0) stf<A>(k_cache + (int64_t)slot * nk + e, v);
   }
-  if (slot >= 0)
+  if (slot >= 0 && G > 0)
     for (int i = threadIdx.x; i < G * Dv; i += NT) v_cache[(int64_t)slot * G * Dv + i] = row[nq + nk + i];
 }
 
@@ -698,8 +698,9 @@ __global__ __launch_bounds__(NT) void sigmoid_route_kernel(const A* __restrict__
 }
 
 // ------------------------------------------------------------------------------------------------ experts, any shape
-// act[p, f] = relu(up[e_p, f, :] · h[t])²  for the routed pair p = t·K + slot
-template <typename A>
+// act[p, f] = relu(up[e_p, f, :] · h[t])²  for the routed pair p = t·K + slot; GATED: an expert's rows are F gate rows, then F
+// up rows, and act[p, f] = silu(gate[e_p, f, :] · h[t]) · (up[e_p, f, :] · h[t])
+template <typename A, bool GATED>
 __global__ __launch_bounds__(NT) void expert_up_kernel(const A* __restrict__ h, int64_t h_stride, const int* __restrict__ ids, int K,
                                                        const A* __restrict__ up, int F, int W, A* __restrict__ act) {
   extern __shared__ float sh[];
@@ -709,10 +710,15 @@ __global__ __launch_bounds__(NT) void expert_up_kernel(const A* __restrict__ h, 
   for (int i = threadIdx.x; i < W; i += NT) sh[i] = ldf<A>(h + t * h_stride + i);
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const A* we = up + (int64_t)e * F * W;
+  const A* we = up + (int64_t)e * (GATED ? 2 : 1) * F * W;
   for (int f = wave; f < F; f += NT / 64) {
-    const float d = fmaxf(wave_dot<A>(sh, we + (int64_t)f * W, W), 0.f);
-    if (lane == 0) stf<A>(act + p * F + f, d * d);
+    if (GATED) {
+      const float g = wave_dot<A>(sh, we + (int64_t)f * W, W), u = wave_dot<A>(sh, we + (int64_t)(F + f) * W, W);
+      if (lane == 0) stf<A>(act + p * F + f, g * sigmoid_f(g) * u);
+    } else {
+      const float d = fmaxf(wave_dot<A>(sh, we + (int64_t)f * W, W), 0.f);
+      if (lane == 0) stf<A>(act + p * F + f, d * d);
+    }
   }
 }
 
@@ -909,11 +915,15 @@ void launch_dm_sigmoid_route(const void* h, bool bf16, int64_t h_stride, const f
 }
 
 void launch_dm_experts(const void* h, bool bf16, int64_t h_stride, const int* ids, const float* wts, int K, const void* up,
-                       const void* down, int rows, int F, int W, void* act, void* out, hipStream_t stream) {
+                       const void* down, int rows, int F, int W, void* act, void* out, bool gated, hipStream_t stream) {
   if (rows == 0) return;
   DM_BF16(bf16, A, {
-    hipLaunchKernelGGL(expert_up_kernel<A>, dim3(rows * K), dim3(NT), W * sizeof(float), stream, (const A*)h, h_stride, ids, K,
-                       (const A*)up, F, W, (A*)act);
+    if (gated)
+      hipLaunchKernelGGL((expert_up_kernel<A, true>), dim3(rows * K), dim3(NT), W * sizeof(float), stream, (const A*)h, h_stride, ids, K,
+                         (const A*)up, F, W, (A*)act);
+    else
+      hipLaunchKernelGGL((expert_up_kernel<A, false>), dim3(rows * K), dim3(NT), W * sizeof(float), stream, (const A*)h, h_stride, ids, K,
+                         (const A*)up, F, W, (A*)act);
     hipLaunchKernelGGL(expert_down_kernel<A>, dim3(rows), dim3(NT), (size_t)K * F * sizeof(float), stream, (const A*)act, ids, wts, K,
                        (const A*)down, F, W, (A*)out);
   });

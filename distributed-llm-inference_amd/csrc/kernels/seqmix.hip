@@ -298,7 +298,7 @@ __global__ __launch_bounds__(NT) void add_ln_kernel(float* __restrict__ x, const
 template <typename G, typename O>
 __global__ __launch_bounds__(NT) void rms_gate_kernel(const float* __restrict__ o, int parts, int64_t part_stride,
                                                       const float* __restrict__ w, float eps, const G* __restrict__ gate,
-                                                      int64_t gate_stride, int N, O* __restrict__ out) {
+                                                      int64_t gate_stride, int N, O* __restrict__ out, int groups, int silu) {
   extern __shared__ float sh[];
   __shared__ float red[NT / 64];
   const int64_t t = blockIdx.x;
@@ -309,10 +309,30 @@ __global__ __launch_bounds__(NT) void rms_gate_kernel(const float* __restrict__ 
     sh[i] = v;
     s += v * v;
   }
-  const float inv = 1.f / sqrtf(block_sum<NT>(s, red) / (float)N + eps);
-  for (int i = threadIdx.x; i < N; i += NT) {
-    const float g = ldf<G>(gate + t * gate_stride + i);
-    stf<O>(out + t * N + i, sh[i] * inv * w[i] / (1.f + expf(-g)));
+  if (groups <= 1) {
+    const float inv = 1.f / sqrtf(block_sum<NT>(s, red) / (float)N + eps);
+    for (int i = threadIdx.x; i < N; i += NT) {
+      const float g = ldf<G>(gate + t * gate_stride + i);
+      const float a = 1.f / (1.f + expf(-g));
+      stf<O>(out + t * N + i, sh[i] * inv * (w != nullptr ? w[i] : 1.f) * (silu ? g * a : a));
+    }
+    return;
+  }
+  // every slice of N / groups entries has its own statistic: a wave per slice
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int Dg = N / groups;
+  for (int gi = wave; gi < groups; gi += NT / 64) {
+    const float* row = sh + gi * Dg;
+    float q = 0.f;
+    for (int i = lane; i < Dg; i += 64) q += row[i] * row[i];
+    const float inv = 1.f / sqrtf(wave_sum(q) / (float)Dg + eps);
+    for (int i = lane; i < Dg; i += 64) {
+      const int c = gi * Dg + i;
+      const float g = ldf<G>(gate + t * gate_stride + c);
+      const float a = 1.f / (1.f + expf(-g));
+      stf<O>(out + t * N + c, row[i] * inv * (w != nullptr ? w[c] : 1.f) * (silu ? g * a : a));
+    }
   }
 }
 
@@ -478,7 +498,7 @@ __global__ __launch_bounds__(NT) void token_attention_kernel(
     const A* __restrict__ vc, int rowv, int vhead, int Dv, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ token_seq, int H, int G, float scale, int window,
     const float* __restrict__ temp, const float* __restrict__ r1, const float* __restrict__ r2, int nsplit,
-    float* __restrict__ part) {
+    float* __restrict__ part, const A* __restrict__ gate, int64_t g_ts) {
   extern __shared__ float sh[];          // q [HG][Dk] | acc [4 waves][HG][Dv] | m [4][HG] | l [4][HG]
   constexpr int NW = NT / 64;
   const int64_t t = blockIdx.x;
@@ -652,7 +672,8 @@ __global__ __launch_bounds__(NT) void token_attention_kernel(
       o += f * accs[(w * HG + hh) * Dv + e];
     }
     if (nsplit == 1) {
-      stf<A>(out + t * o_ts + (h0 + hh) * o_hs + e, o / L);
+      const float gm = gate != nullptr ? 1.f / (1.f + expf(-ldf<A>(gate + t * g_ts + h0 + hh))) : 1.f;
+      stf<A>(out + t * o_ts + (h0 + hh) * o_hs + e, o / L * gm);
     } else {
       float* pr = part + ((t * H + (h0 + hh)) * nsplit + blockIdx.z) * (int64_t)(Dv + 2);
       pr[2 + e] = o;
@@ -669,7 +690,7 @@ template <typename A>
 __global__ __launch_bounds__(128) void token_attention_merge_kernel(A* __restrict__ out, int64_t o_ts, int64_t o_hs,
                                                                     const float* __restrict__ part,
                                                                     const int* __restrict__ token_seq, int H, int Dv,
-                                                                    int nsplit) {
+                                                                    int nsplit, const A* __restrict__ gate, int64_t g_ts) {
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y;
   if (token_seq[t] < 0) return;
@@ -684,7 +705,7 @@ __global__ __launch_bounds__(128) void token_attention_merge_kernel(A* __restric
     f[z] = mz == -INFINITY ? 0.f : expf(mz - M);
     if (z < nsplit) L += f[z] * pr[z * (Dv + 2) + 1];
   }
-  const float rl = 1.f / L;
+  const float rl = (gate != nullptr ? 1.f / (1.f + expf(-ldf<A>(gate + t * g_ts + h))) : 1.f) / L;
   for (int e = threadIdx.x; e < Dv; e += 128) {
     float o = 0.f;
 #pragma unroll
@@ -710,7 +731,8 @@ __global__ __launch_bounds__(NT * HW) void tile_attention_kernel(
     const uint16_t* __restrict__ vc, int rowv, int vhead, int Dv, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ seq_lens, const int* __restrict__ qsl, const int* __restrict__ tile_seq,
     const int* __restrict__ tile_q0, int num_tiles, const int* __restrict__ counts, int H, int G, float scale, int window,
-    const float* __restrict__ temp, const float* __restrict__ r1, const float* __restrict__ r2) {
+    const float* __restrict__ temp, const float* __restrict__ r1, const float* __restrict__ r2,
+    const uint16_t* __restrict__ gate, int64_t g_ts) {
   extern __shared__ __align__(16) uint16_t tl[];
   const int ntiles = counts != nullptr ? min(counts[2], num_tiles) : num_tiles;
   // the host walks causal tiles longest-first from the END of the list
@@ -850,7 +872,7 @@ __global__ __launch_bounds__(NT * HW) void tile_attention_kernel(
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!qvalid) return;
-  const float rl = 1.f / l;
+  const float rl = (gate != nullptr ? 1.f / (1.f + expf(-bf2f(gate[tq * g_ts + h]))) : 1.f) / l;
   uint16_t* orow = out + tq * o_ts + h * o_hs;
 #pragma unroll
   for (int i = 0; i < MTMAX; ++i) {
@@ -877,7 +899,7 @@ __global__ __launch_bounds__(NT) void head_decode_attention_kernel(
     const uint16_t* __restrict__ vc, int rowv, int vhead, int Dv, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ token_seq, int H, int G, int groups, float scale, int window,
     const float* __restrict__ temp, const float* __restrict__ r1, const float* __restrict__ r2, int nsplit,
-    float* __restrict__ part) {
+    float* __restrict__ part, const uint16_t* __restrict__ gate, int64_t g_ts) {
   extern __shared__ __align__(16) uint16_t tl[];
   const int64_t t = blockIdx.x;
   const int seq = token_seq[t];
@@ -997,7 +1019,7 @@ __global__ __launch_bounds__(NT) void head_decode_attention_kernel(
   l += __shfl_xor(l, 32, 64);
   if (!hvalid) return;
   if (nsplit == 1) {
-    const float rl = 1.f / l;
+    const float rl = (gate != nullptr ? 1.f / (1.f + expf(-bf2f(gate[t * g_ts + h]))) : 1.f) / l;
     uint16_t* orow = out + t * o_ts + h * o_hs;
 #pragma unroll
     for (int ii = 0; ii < MTQ; ++ii) {
@@ -1028,7 +1050,8 @@ __global__ __launch_bounds__(NT) void head_decode_attention_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------ linear attention
-// S ← decay·S + silu(k)·silu(v)ᵀ, o = Sᵀ silu(q), token by token, with S = a [D, Dv] fp32 state per (sequence, head).
+// S ← decay·S + act(k)·act(v)ᵀ, o = Sᵀ act(q), token by token, with S = a [D, Dv] fp32 state per (sequence, head); act is
+// silu, or the identity with `plain` (retention: q and k arrive rotated and scaled, in fp32).
 // One wave per (work item, head, 64 value columns): lane e keeps column e of the state in registers; the next token's
 // q / k / v are fetched while the current one is applied.  DMAX: compile-time bound of D (registers per lane).
 //
@@ -1049,7 +1072,7 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict_
                                                             const float* __restrict__ decay, float* __restrict__ out,
                                                             const int* __restrict__ tile_seq, const int* __restrict__ tile_q0,
                                                             int num_tiles, float* __restrict__ ws, int single_only, int zs,
-                                                            int DR, int64_t out_part) {
+                                                            int DR, int64_t out_part, int plain) {
   __shared__ float qs[2][DMAX], ks[2][DMAX];
   int seq, t0, t1;
   if (MODE == 0) {
@@ -1107,11 +1130,11 @@ __global__ __launch_bounds__(64) void lightning_scan_kernel(const A* __restrict_
     for (int r = 0; r < PER; ++r) {
       const int i = lane + 64 * r;
       if (i < DMAX) {
-        if (MODE != 1) qs[buf][i] = silu_act<A>(nq[r]);
-        ks[buf][i] = silu_act<A>(nk[r]);
+        if (MODE != 1) qs[buf][i] = plain ? nq[r] : silu_act<A>(nq[r]);
+        ks[buf][i] = plain ? nk[r] : silu_act<A>(nk[r]);
       }
     }
-    const float ve = silu_act<A>(nv);
+    const float ve = plain ? nv : silu_act<A>(nv);
     if (t + 1 < t1) fetch(t + 1);
     __syncthreads();                       // one wave: publishes qs / ks of this token (the other buffer is being refilled next trip)
     float o = 0.f;
@@ -1209,12 +1232,13 @@ void launch_sm_add_ln(float* x, const void* y, bool y_bf16, int64_t y_stride, co
 }
 
 void launch_sm_rms_gate(const float* o, int parts, const float* w, float eps, const void* gate, bool gate_bf16, int64_t gate_stride,
-                        int rows, int N, void* out, bool out_bf16, hipStream_t stream) {
+                        int rows, int N, void* out, bool out_bf16, int groups, bool silu, hipStream_t stream) {
   if (rows == 0) return;
   const int64_t ps = (int64_t)rows * N;
   SM_DISPATCH_BF16(gate_bf16, G, SM_DISPATCH_BF16(out_bf16, O, hipLaunchKernelGGL((rms_gate_kernel<G, O>), dim3(rows), dim3(NT),
                                                                                    N * sizeof(float), stream, o, parts, ps, w, eps,
-                                                                                   (const G*)gate, gate_stride, N, (O*)out)));
+                                                                                   (const G*)gate, gate_stride, N, (O*)out, groups,
+                                                                                   silu ? 1 : 0)));
 }
 
 void launch_sm_relu2(const void* x, void* out, int64_t n, bool bf16, hipStream_t stream) {
@@ -1251,11 +1275,11 @@ static void token_attention_hg(int hg, dim3 grid, size_t lds, hipStream_t stream
                                int64_t q1_ts, int64_t q1_hs, int D1, const A* q2, int64_t q2_ts, int64_t q2_hs, int D2, const A* kc,
                                int rowk, const A* vc, int rowv, int vhead, int Dv, const int* bt, int max_blocks, const int* pos,
                                const int* tseq, int H, int G, float scale, int window, const float* temp, const float* r1,
-                               const float* r2, int nsplit, float* part) {
+                               const float* r2, int nsplit, float* part, const A* gate, int64_t g_ts) {
 #define SM_ATT(HGV)                                                                                                              \
   hipLaunchKernelGGL((token_attention_kernel<A, VPL, HGV>), grid, dim3(NT), lds, stream, out, o_ts, o_hs, q1, q1_ts, q1_hs, D1,  \
                      q2, q2_ts, q2_hs, D2, kc, rowk, vc, rowv, vhead, Dv, bt, max_blocks, pos, tseq, H, G, scale, window, temp,  \
-                     r1, r2, nsplit, part)
+                     r1, r2, nsplit, part, gate, g_ts)
   if (hg == 1) SM_ATT(1);
   else if (hg == 2) SM_ATT(2);
   else SM_ATT(4);
@@ -1266,7 +1290,8 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
                                const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
                                int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* positions,
                                const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
-                               const float* r1, const float* r2, bool bf16, int nsplit, float* part, hipStream_t stream) {
+                               const float* r1, const float* r2, bool bf16, int nsplit, float* part, const void* gate, int64_t g_ts,
+                               hipStream_t stream) {
   if (rows == 0) return;
   if (Dv > 512) {
     // wider values than a lane's 8 columns × 64 lanes: slabs of 512 columns, each a launch of its own (scores recomputed)
@@ -1274,7 +1299,7 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
       launch_sm_token_attention(bf16 ? (void*)((uint16_t*)out + e) : (void*)((float*)out + e), o_ts, o_hs, q1, q1_ts, q1_hs, D1, q2,
                                 q2_ts, q2_hs, D2, kc, rowk, bf16 ? (const void*)((const uint16_t*)vc + e) : (const void*)((const float*)vc + e),
                                 rowv, vhead, std::min(512, Dv - e), block_tables, max_blocks, positions, token_seq, rows, H, G, scale,
-                                window, temp, r1, r2, bf16, 1, nullptr, stream);
+                                window, temp, r1, r2, bf16, 1, nullptr, gate, g_ts, stream);
     return;
   }
   // heads per workgroup: as many of the heads sharing a key / value head as divide their number and fit the LDS budget
@@ -1289,7 +1314,7 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
   SM_DISPATCH_BF16(bf16, A, (token_attention_hg<A, VPLV>(hg, grid, lds, stream, (A*)out, o_ts, o_hs, (const A*)q1, q1_ts, q1_hs, \
                                                          D1, (const A*)q2, q2_ts, q2_hs, D2, (const A*)kc, rowk, (const A*)vc,   \
                                                          rowv, vhead, Dv, block_tables, max_blocks, positions, token_seq, H, G,  \
-                                                         scale, window, temp, r1, r2, nsplit, part)))
+                                                         scale, window, temp, r1, r2, nsplit, part, (const A*)gate, g_ts)))
   if (nv <= 1) SM_ATT_V(1);
   else if (nv <= 2) SM_ATT_V(2);
   else if (nv <= 4) SM_ATT_V(4);
@@ -1297,7 +1322,7 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
 #undef SM_ATT_V
   if (nsplit > 1)
     SM_DISPATCH_BF16(bf16, A, hipLaunchKernelGGL(token_attention_merge_kernel<A>, dim3(rows, H), dim3(128), 0, stream, (A*)out, o_ts,
-                                                 o_hs, (const float*)part, token_seq, H, Dv, nsplit));
+                                                 o_hs, (const float*)part, token_seq, H, Dv, nsplit, (const A*)gate, g_ts));
 }
 
 // workgroups of a per-token attention launch over `rows` tokens: long key ranges are cut so that about 1024 exist
@@ -1315,7 +1340,7 @@ bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void*
                               int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* seq_lens,
                               const int* qsl, const int* tile_seq, const int* tile_q0, int num_tiles, const int* counts, int H,
                               int G, float scale, int window, const float* temp, const float* r1, const float* r2,
-                              hipStream_t stream) {
+                              const void* gate, int64_t g_ts, hipStream_t stream) {
   const int Dk = D1 + D2, KS = (Dk + 31) / 32, MT = Dv / 16;
   auto al = [](const void* p, int64_t a) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % a == 0; };
   const bool ok = D1 % 8 == 0 && D2 % 8 == 0 && Dv % 16 == 0 && KS <= 18 && MT <= 32 && rowk % 8 == 0 && rowv % 8 == 0 &&
@@ -1338,7 +1363,7 @@ bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void*
     hipLaunchKernelGGL((tile_attention_kernel<KSM, MTM, HWV>), grid, dim3(NT * HWV), lds, stream, (uint16_t*)out, o_ts, o_hs,    \
                        (const uint16_t*)q1, q1_ts, q1_hs, D1, (const uint16_t*)q2, q2_ts, q2_hs, D2, (const uint16_t*)kc, rowk,  \
                        (const uint16_t*)vc, rowv, vhead, Dv, block_tables, max_blocks, seq_lens, qsl, tile_seq, tile_q0,        \
-                       num_tiles, counts, H, G, scale, window, temp, r1, r2);                                                    \
+                       num_tiles, counts, H, G, scale, window, temp, r1, r2, (const uint16_t*)gate, g_ts);                       \
   } while (0)
 #define SM_TILE(KSM, MTM)              \
   do {                                 \
@@ -1358,7 +1383,8 @@ bool launch_sm_head_decode_attention(void* out, int64_t o_ts, int64_t o_hs, cons
                                      const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
                                      int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* positions,
                                      const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
-                                     const float* r1, const float* r2, int nsplit, float* part, hipStream_t stream) {
+                                     const float* r1, const float* r2, int nsplit, float* part, const void* gate, int64_t g_ts,
+                                     hipStream_t stream) {
   const int Dk = D1 + D2, KS = (Dk + 31) / 32, MT = Dv / 16, per = H / G;
   auto al = [](const void* p, int64_t a) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % a == 0; };
   const bool ok = per >= 8 && D1 % 8 == 0 && D2 % 8 == 0 && Dv % 16 == 0 && KS <= 18 && MT <= 32 && rowk % 8 == 0 && rowv % 8 == 0 &&
@@ -1380,7 +1406,7 @@ bool launch_sm_head_decode_attention(void* out, int64_t o_ts, int64_t o_hs, cons
     hipLaunchKernelGGL((head_decode_attention_kernel<KSM, MTQV>), grid, dim3(NT), lds, stream, (uint16_t*)out, o_ts, o_hs,       \
                        (const uint16_t*)q1, q1_ts, q1_hs, D1, (const uint16_t*)q2, q2_ts, q2_hs, D2, (const uint16_t*)kc, rowk,  \
                        (const uint16_t*)vc, rowv, vhead, Dv, block_tables, max_blocks, positions, token_seq, H, G, groups, scale,\
-                       window, temp, r1, r2, nsplit, part);                                                                      \
+                       window, temp, r1, r2, nsplit, part, (const uint16_t*)gate, g_ts);                                         \
   } while (0)
   if (KS <= 4 && MT <= 8) SM_HD(4, 2);
   else if (KS <= 8 && MT <= 16) SM_HD(8, 4);
@@ -1388,7 +1414,7 @@ bool launch_sm_head_decode_attention(void* out, int64_t o_ts, int64_t o_hs, cons
 #undef SM_HD
   if (nsplit > 1)
     hipLaunchKernelGGL(token_attention_merge_kernel<uint16_t>, dim3(rows, H), dim3(128), 0, stream, (uint16_t*)out, o_ts, o_hs,
-                       (const float*)part, token_seq, H, Dv, nsplit);
+                       (const float*)part, token_seq, H, Dv, nsplit, (const uint16_t*)gate, g_ts);
   return true;
 }
 
@@ -1405,27 +1431,28 @@ int sm_lightning_parts(int D) { return D >= 128 ? 4 : (D >= 64 ? 2 : 1); }
 void launch_sm_lightning_scan(const void* qkvg, bool bf16, int64_t row_stride, float* state, const int* positions, const int* qsl,
                               const int* state_slots, const int* counts, int seqs, int H, int D, int Dv, const float* decay,
                               float* out, int64_t out_part, const int* tile_seq, const int* tile_q0, int num_tiles, float* ws,
-                              hipStream_t stream) {
+                              bool plain_act, hipStream_t stream) {
   if (seqs == 0) return;
   const int zs = (Dv + 63) / 64;
   const int parts = sm_lightning_parts(D);
   const int DR = (D + parts - 1) / parts;
   const unsigned gz = zs * parts;
   const bool blocks = num_tiles > 0 && ws != nullptr;
+  const int plain = plain_act ? 1 : 0;
 #define SM_SCAN(DM)                                                                                                                  \
   SM_DISPATCH_BF16(bf16, A, {                                                                                                         \
     hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 0>), dim3(seqs, H, gz), dim3(64), 0, stream, (const A*)qkvg, row_stride, state,  \
                        positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, blocks ? 1 : 0,  \
-                       zs, DR, out_part);                                                                                            \
+                       zs, DR, out_part, plain);                                                                                     \
     if (blocks) {                                                                                                                    \
       hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 1>), dim3(num_tiles, H, gz), dim3(64), 0, stream, (const A*)qkvg, row_stride,  \
                          state, positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, 0, zs,  \
-                         DR, out_part);                                                                                              \
+                         DR, out_part, plain);                                                                                       \
       hipLaunchKernelGGL(lightning_prefix_kernel, dim3(seqs, H, zs * D), dim3(64), 0, stream, state, ws, positions, qsl, state_slots, \
                          counts, H, D, Dv, decay);                                                                                   \
       hipLaunchKernelGGL((lightning_scan_kernel<A, DM, 2>), dim3(num_tiles, H, gz), dim3(64), 0, stream, (const A*)qkvg, row_stride,  \
                          state, positions, qsl, state_slots, counts, H, D, Dv, decay, out, tile_seq, tile_q0, num_tiles, ws, 0, zs,  \
-                         DR, out_part);                                                                                              \
+                         DR, out_part, plain);                                                                                       \
     }                                                                                                                                \
   })
   if (DR <= 32) SM_SCAN(32);

@@ -91,19 +91,21 @@ Tensor sm_add_ln(Tensor x, const Tensor& y, const Tensor& w, const Tensor& b, do
   return out;
 }
 
-Tensor sm_rms_gate(const Tensor& o, const Tensor& w, double eps, const Tensor& gate, bool out_bf16) {
+Tensor sm_rms_gate(const Tensor& o, const c10::optional<Tensor>& w, double eps, const Tensor& gate, bool out_bf16, int64_t groups,
+                   bool silu) {
   check_f32(o, "o");
   TORCH_CHECK(o.dim() == 2 || o.dim() == 3, "o must be [T, N] or planes of partial sums [parts, T, N]");
   const int64_t parts = o.dim() == 3 ? o.size(0) : 1;
   const int64_t T = o.size(-2), N = o.size(-1);
   TORCH_CHECK(N * 4 <= kSmMaxLds, "row too wide");
-  check_f32(w, "w", N);
+  const float* wp = opt_f32(w, "w", N);
+  TORCH_CHECK(groups >= 1 && N % groups == 0, "the row does not divide into that many groups");
   const bool gbf = act_bf16(gate, "gate");
   check_rows(gate, "gate");
   TORCH_CHECK(gate.size(0) == T && gate.size(1) == N, "gate must be [T, N]");
   Tensor out = at::empty({T, N}, o.options().dtype(out_bf16 ? at::kBFloat16 : at::kFloat));
-  dli::launch_sm_rms_gate(o.data_ptr<float>(), (int)parts, w.data_ptr<float>(), (float)eps, gate.data_ptr(), gbf, gate.stride(0), (int)T,
-                          (int)N, out.data_ptr(), out_bf16, cur_stream(o));
+  dli::launch_sm_rms_gate(o.data_ptr<float>(), (int)parts, wp, (float)eps, gate.data_ptr(), gbf, gate.stride(0), (int)T, (int)N,
+                          out.data_ptr(), out_bf16, (int)groups, silu, cur_stream(o));
   return out;
 }
 
@@ -165,10 +167,21 @@ void sm_latent_prep(Tensor q, const Tensor& dkv, const Tensor& cw, double eps, c
                              cache.data_ptr(), (int)T, (int)H, (int)D, (int)R, (int)C, cur_stream(q));
 }
 
+// per-head output gate of the attention kernels: [T, H] rows (pre-activation, row-strided view) of the queries' dtype
+const void* head_gate(const c10::optional<Tensor>& gate, const Tensor& q1, int64_t T, int64_t H, int64_t* stride) {
+  *stride = 0;
+  if (!gate.has_value()) return nullptr;
+  TORCH_CHECK(gate->is_cuda() && gate->scalar_type() == q1.scalar_type() && gate->dim() == 2 && gate->stride(1) == 1 &&
+                  gate->size(0) == T && gate->size(1) == H, "gate must be [T, H] like the queries");
+  *stride = gate->stride(0);
+  return gate->data_ptr();
+}
+
 void sm_token_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor>& q2, const Tensor& k_cache,
                         const c10::optional<Tensor>& v_cache, const Tensor& block_tables, const Tensor& positions,
                         const Tensor& token_seq, int64_t G, int64_t Dv, double scale, int64_t window, const c10::optional<Tensor>& temp,
-                        const c10::optional<Tensor>& r1, const c10::optional<Tensor>& r2, int64_t rows) {
+                        const c10::optional<Tensor>& r1, const c10::optional<Tensor>& r2, int64_t rows,
+                        const c10::optional<Tensor>& gate) {
   const bool bf = act_bf16(q1, "q1");
   TORCH_CHECK(q1.dim() == 3 && q1.stride(2) == 1, "q1 must be [T, H, D1] with a contiguous last dim");
   TORCH_CHECK(rows < 0 || rows <= q1.size(0), "rows past the batch");
@@ -201,6 +214,8 @@ void sm_token_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor
   TORCH_CHECK(block_tables.dim() == 2 && positions.numel() >= T && token_seq.numel() >= T, "step metadata shorter than the batch");
   TORCH_CHECK(r1.has_value() == r2.has_value(), "r1 and r2 come together");
   TORCH_CHECK((Dk + 4 * std::min<int64_t>(Dv, 512) + 8) * 4 <= kSmMaxLds, "head sizes exceed the kernel's LDS budget");
+  int64_t g_ts = 0;
+  const void* gp = head_gate(gate, q1, T, H, &g_ts);
   // few rows (decode steps): long key ranges are cut over several workgroups, partial results in `part`
   const int64_t n_rows = rows < 0 ? T : rows;
   const int nsplit = Dv > 512 ? 1 : dli::sm_token_attention_splits((int)n_rows, (int)H, (int)G);
@@ -212,7 +227,7 @@ void sm_token_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor
                                  (int)vc.size(2), (int)vhead, (int)Dv, block_tables.data_ptr<int>(), (int)block_tables.size(1),
                                  positions.data_ptr<int>(), token_seq.data_ptr<int>(), (int)n_rows, (int)H, (int)G, (float)scale,
                                  (int)window, opt_f32(temp, "temp", H), opt_f32(r1, "r1", H), opt_f32(r2, "r2", H), bf, nsplit,
-                                 nsplit > 1 ? part.data_ptr<float>() : nullptr, cur_stream(q1));
+                                 nsplit > 1 ? part.data_ptr<float>() : nullptr, gp, g_ts, cur_stream(q1));
 }
 
 // Decode rows (the first `rows` tokens) of a mixer whose heads share key / value heads in groups of 8 or more, heads as the
@@ -221,7 +236,7 @@ bool sm_head_decode_attention(Tensor out, const Tensor& q1, const c10::optional<
                               const c10::optional<Tensor>& v_cache, const Tensor& block_tables, const Tensor& positions,
                               const Tensor& token_seq, int64_t G, int64_t Dv, double scale, int64_t window,
                               const c10::optional<Tensor>& temp, const c10::optional<Tensor>& r1, const c10::optional<Tensor>& r2,
-                              int64_t rows) {
+                              int64_t rows, const c10::optional<Tensor>& gate) {
   TORCH_CHECK(q1.is_cuda() && q1.scalar_type() == at::kBFloat16 && q1.dim() == 3 && q1.stride(2) == 1, "q1 must be bfloat16 [T, H, D1]");
   const int64_t T = q1.size(0), H = q1.size(1), D1 = q1.size(2);
   TORCH_CHECK(rows >= 0 && rows <= T, "rows past the batch");
@@ -251,6 +266,8 @@ bool sm_head_decode_attention(Tensor out, const Tensor& q1, const c10::optional<
   check_i32(token_seq, "token_seq");
   TORCH_CHECK(block_tables.dim() == 2 && positions.numel() >= T && token_seq.numel() >= T, "step metadata shorter than the batch");
   TORCH_CHECK(r1.has_value() == r2.has_value(), "r1 and r2 come together");
+  int64_t g_ts = 0;
+  const void* gp = head_gate(gate, q1, T, H, &g_ts);
   const int nsplit = dli::sm_head_decode_splits((int)rows, (int)H, (int)G);
   Tensor part;
   if (nsplit > 1) part = at::empty({std::max<int64_t>(rows, 1), H, nsplit, Dv + 2}, q1.options().dtype(at::kFloat));
@@ -260,7 +277,8 @@ bool sm_head_decode_attention(Tensor out, const Tensor& q1, const c10::optional<
                                               vc.data_ptr(), (int)vc.size(2), (int)vhead, (int)Dv, block_tables.data_ptr<int>(),
                                               (int)block_tables.size(1), positions.data_ptr<int>(), token_seq.data_ptr<int>(), (int)rows,
                                               (int)H, (int)G, (float)scale, (int)window, opt_f32(temp, "temp", H), opt_f32(r1, "r1", H),
-                                              opt_f32(r2, "r2", H), nsplit, nsplit > 1 ? part.data_ptr<float>() : nullptr, cur_stream(q1));
+                                              opt_f32(r2, "r2", H), nsplit, nsplit > 1 ? part.data_ptr<float>() : nullptr, gp, g_ts,
+                                              cur_stream(q1));
 }
 
 // Prefill tiles (64 queries of one sequence's chunk each) on the matrix cores; bf16 only.  False: shapes the tile kernel does
@@ -269,7 +287,7 @@ bool sm_tile_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor>
                        const c10::optional<Tensor>& v_cache, const Tensor& block_tables, const Tensor& seq_lens, const Tensor& qsl,
                        const Tensor& tile_seq, const Tensor& tile_q0, int64_t num_tiles, const c10::optional<Tensor>& counts, int64_t G,
                        int64_t Dv, double scale, int64_t window, const c10::optional<Tensor>& temp, const c10::optional<Tensor>& r1,
-                       const c10::optional<Tensor>& r2) {
+                       const c10::optional<Tensor>& r2, const c10::optional<Tensor>& gate) {
   TORCH_CHECK(q1.is_cuda() && q1.scalar_type() == at::kBFloat16 && q1.dim() == 3 && q1.stride(2) == 1, "q1 must be bfloat16 [T, H, D1]");
   const int64_t T = q1.size(0), H = q1.size(1), D1 = q1.size(2);
   int64_t D2 = 0;
@@ -307,18 +325,21 @@ bool sm_tile_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor>
     cnt = counts->data_ptr<int>();
   }
   TORCH_CHECK(r1.has_value() == r2.has_value(), "r1 and r2 come together");
+  int64_t g_ts = 0;
+  const void* gp = head_gate(gate, q1, T, H, &g_ts);
   return dli::launch_sm_tile_attention(out.data_ptr(), out.stride(0), out.stride(1), q1.data_ptr(), q1.stride(0), q1.stride(1), (int)D1,
                                        q2.has_value() ? q2->data_ptr() : nullptr, q2.has_value() ? q2->stride(0) : 0,
                                        q2.has_value() ? q2->stride(1) : 0, (int)D2, k_cache.data_ptr(), (int)(G * Dk), vc.data_ptr(),
                                        (int)vc.size(2), (int)vhead, (int)Dv, block_tables.data_ptr<int>(), (int)block_tables.size(1),
                                        seq_lens.data_ptr<int>(), qsl.data_ptr<int>(), tile_seq.data_ptr<int>(), tile_q0.data_ptr<int>(),
                                        (int)num_tiles, cnt, (int)H, (int)G, (float)scale, (int)window, opt_f32(temp, "temp", H),
-                                       opt_f32(r1, "r1", H), opt_f32(r2, "r2", H), cur_stream(q1));
+                                       opt_f32(r1, "r1", H), opt_f32(r2, "r2", H), gp, g_ts, cur_stream(q1));
 }
 
 Tensor sm_lightning_scan(const Tensor& qkvg, Tensor state, const Tensor& positions, const Tensor& qsl, const Tensor& state_slots,
                          const Tensor& counts, int64_t num_seqs, int64_t H, int64_t D, int64_t Dv, const Tensor& decay,
-                         const c10::optional<Tensor>& tile_seq, const c10::optional<Tensor>& tile_q0, int64_t num_tiles) {
+                         const c10::optional<Tensor>& tile_seq, const c10::optional<Tensor>& tile_q0, int64_t num_tiles,
+                         bool plain_act) {
   const bool bf = act_bf16(qkvg, "qkvg");
   check_rows(qkvg, "qkvg");
   const int64_t T = qkvg.size(0);
@@ -352,6 +373,6 @@ Tensor sm_lightning_scan(const Tensor& qkvg, Tensor state, const Tensor& positio
   dli::launch_sm_lightning_scan(qkvg.data_ptr(), bf, qkvg.stride(0), state.data_ptr<float>(), positions.data_ptr<int>(),
                                 qsl.data_ptr<int>(), state_slots.data_ptr<int>(), counts.data_ptr<int>(), (int)num_seqs, (int)H, (int)D,
                                 (int)Dv, decay.data_ptr<float>(), out.data_ptr<float>(), T * H * Dv, ts, tq, (int)num_tiles,
-                                num_tiles > 0 ? ws.data_ptr<float>() : nullptr, cur_stream(qkvg));
+                                num_tiles > 0 ? ws.data_ptr<float>() : nullptr, plain_act, cur_stream(qkvg));
   return out;
 }

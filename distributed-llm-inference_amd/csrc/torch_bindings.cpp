@@ -575,6 +575,7 @@ void ar_all_gather(int64_t st, const Tensor& inp, Tensor out) {
 
 #include "seqmix_bindings.h"
 #include "dualmix_bindings.h"
+#include "hypermix_bindings.h"
 
 }  // namespace
 
@@ -584,7 +585,7 @@ TORCH_LIBRARY(dli, m) {
         "Tensor token_seq, Tensor qsl, Tensor state_slots, Tensor counts, int num_seqs, bool out_bf16) -> (Tensor, Tensor)", &sm_ln_shift);
   m.def("sm_add_ln(Tensor(a!) x, Tensor y, Tensor w, Tensor b, float eps, float mult, Tensor? w2, Tensor? b2, bool out_bf16) -> Tensor",
         &sm_add_ln);
-  m.def("sm_rms_gate(Tensor o, Tensor w, float eps, Tensor gate, bool out_bf16) -> Tensor", &sm_rms_gate);
+  m.def("sm_rms_gate(Tensor o, Tensor? w, float eps, Tensor gate, bool out_bf16, int groups=1, bool silu=False) -> Tensor", &sm_rms_gate);
   m.def("sm_relu2(Tensor x) -> Tensor", &sm_relu2);
   m.def("sm_softcap(Tensor x, float cap) -> Tensor", &sm_softcap);
   m.def("sm_qk_norm_cache(Tensor(a!) qkv, Tensor qw, Tensor kw, float eps, Tensor slot_mapping, Tensor(b!) k_cache, Tensor(c!) v_cache, "
@@ -592,22 +593,24 @@ TORCH_LIBRARY(dli, m) {
   m.def("sm_latent_prep(Tensor(a!) q, Tensor dkv, Tensor cw, float eps, Tensor positions, Tensor inv_freq, int rot_dims, "
         "Tensor slot_mapping, Tensor(b!) cache, int H, int D, int R, int C) -> ()", &sm_latent_prep);
   m.def("sm_token_attention(Tensor(a!) out, Tensor q1, Tensor? q2, Tensor k_cache, Tensor? v_cache, Tensor block_tables, "
-        "Tensor positions, Tensor token_seq, int G, int Dv, float scale, int window, Tensor? temp, Tensor? r1, Tensor? r2, int rows=-1) -> ()",
+        "Tensor positions, Tensor token_seq, int G, int Dv, float scale, int window, Tensor? temp, Tensor? r1, Tensor? r2, int rows=-1, "
+        "Tensor? gate=None) -> ()",
         &sm_token_attention);
   m.def("sm_head_decode_attention(Tensor(a!) out, Tensor q1, Tensor? q2, Tensor k_cache, Tensor? v_cache, Tensor block_tables, "
-        "Tensor positions, Tensor token_seq, int G, int Dv, float scale, int window, Tensor? temp, Tensor? r1, Tensor? r2, int rows) -> bool",
+        "Tensor positions, Tensor token_seq, int G, int Dv, float scale, int window, Tensor? temp, Tensor? r1, Tensor? r2, int rows, "
+        "Tensor? gate=None) -> bool",
         &sm_head_decode_attention);
   m.def("sm_tile_attention(Tensor(a!) out, Tensor q1, Tensor? q2, Tensor k_cache, Tensor? v_cache, Tensor block_tables, Tensor seq_lens, "
         "Tensor qsl, Tensor tile_seq, Tensor tile_q0, int num_tiles, Tensor? counts, int G, int Dv, float scale, int window, "
-        "Tensor? temp, Tensor? r1, Tensor? r2) -> bool", &sm_tile_attention);
+        "Tensor? temp, Tensor? r1, Tensor? r2, Tensor? gate=None) -> bool", &sm_tile_attention);
   m.def("sm_lightning_scan(Tensor qkvg, Tensor(a!) state, Tensor positions, Tensor qsl, Tensor state_slots, Tensor counts, "
-        "int num_seqs, int H, int D, int Dv, Tensor decay, Tensor? tile_seq=None, Tensor? tile_q0=None, int num_tiles=0) -> Tensor",
-        &sm_lightning_scan);
+        "int num_seqs, int H, int D, int Dv, Tensor decay, Tensor? tile_seq=None, Tensor? tile_q0=None, int num_tiles=0, "
+        "bool plain_act=False) -> Tensor", &sm_lightning_scan);
   m.def("dm_rms_scale(Tensor x, Tensor g1, Tensor? g2, float eps, bool out_bf16) -> (Tensor, Tensor)", &dm_rms_scale);
   m.def("dm_shift_mix(Tensor h, Tensor mu, Tensor(a!) state, Tensor positions, Tensor token_seq, Tensor qsl, Tensor state_slots, "
         "Tensor counts, int num_seqs) -> Tensor", &dm_shift_mix);
-  m.def("dm_wide_norm_rope_cache(Tensor(a!) qkv, Tensor qw, Tensor kw, float eps, Tensor positions, Tensor freq, float mag, int rot_dims, "
-        "Tensor slot_mapping, Tensor(b!) k_cache, Tensor(c!) v_cache, int H, int G, int D, int Dv) -> ()", &dm_wide_norm_rope_cache);
+  m.def("dm_wide_norm_rope_cache(Tensor(a!) qkv, Tensor qw, Tensor? kw, float eps, Tensor positions, Tensor? freq, float mag, int rot_dims, "
+        "Tensor slot_mapping, Tensor(b!)? k_cache, Tensor(c!)? v_cache, int H, int G, int D, int Dv) -> ()", &dm_wide_norm_rope_cache);
   m.def("dm_talk_attention(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor v_cache, Tensor block_tables, Tensor positions, "
         "Tensor token_seq, Tensor? sink, Tensor? talk, int G, int Dv, float scale, int rows=-1) -> ()", &dm_talk_attention);
   m.def("dm_talk_tile_attention(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor v_cache, Tensor block_tables, "
@@ -619,7 +622,15 @@ TORCH_LIBRARY(dli, m) {
         "int num_seqs, int H, int D) -> Tensor", &dm_wkv_scan);
   m.def("dm_group_rms_gate(Tensor o, int groups, Tensor w, float eps, Tensor gate, bool out_bf16) -> Tensor", &dm_group_rms_gate);
   m.def("dm_sigmoid_route(Tensor h, Tensor router, int E, int K, float scale) -> (Tensor, Tensor, Tensor)", &dm_sigmoid_route);
-  m.def("dm_relu2_experts(Tensor h, Tensor ids, Tensor wts, Tensor up, Tensor down) -> Tensor", &dm_relu2_experts);
+  m.def("dm_relu2_experts(Tensor h, Tensor ids, Tensor wts, Tensor up, Tensor down, bool gated=False) -> Tensor", &dm_relu2_experts);
+  m.def("hm_stream_mix_norm(Tensor(a!) x, Tensor? y, Tensor? mix, Tensor? out_w, Tensor? in_w, Tensor? norm_w, float eps, float w_offset, "
+        "bool out_bf16) -> Tensor", &hm_stream_mix_norm);
+  m.def("hm_causal_conv_add(Tensor h, Tensor w, Tensor(a!) state, Tensor positions, Tensor token_seq, Tensor qsl, Tensor state_slots, "
+        "Tensor counts, int num_seqs, bool out_bf16) -> Tensor", &hm_causal_conv_add);
+  m.def("hm_retention_prep(Tensor qkvg, Tensor positions, Tensor? freq, int rot_dims, int H, int D, int Dv, float k_scale) -> Tensor",
+        &hm_retention_prep);
+  m.def("hm_act_mul(Tensor x, bool silu) -> Tensor", &hm_act_mul);
+  m.def("hm_softmax_route(Tensor h, Tensor router, Tensor? bias, int K) -> (Tensor, Tensor)", &hm_softmax_route);
   m.def("dm_relu2_rows(Tensor x) -> Tensor", &dm_relu2_rows);
   m.def("dm_set_grouped_experts(bool on) -> ()", &dm_set_grouped_experts);
   m.def("dm_gated_combine(Tensor(a!) x, float mult, Tensor p0, Tensor p1, float s0, float s1, Tensor g1, Tensor b1, Tensor? ff, "

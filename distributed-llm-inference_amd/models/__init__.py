@@ -102,6 +102,17 @@ class _Shards:
             raise KeyError(f"tensor {key!r} not found in checkpoint")
         return self.where[key].get_tensor(key)
 
+    def cat(self, keys) -> torch.Tensor:
+        """The named tensors concatenated along dim 0; ``"@zeros:<n>"`` stands for ``n`` rows of zeros (rows a fused
+        parameter carries for alignment only)."""
+        real = [self.get(k) for k in keys if not k.startswith("@zeros:")]
+        if len(real) == len(keys):
+            return torch.cat(real, dim=0) if len(real) > 1 else real[0]
+        it = iter(real)
+        parts = [torch.zeros((int(k.split(":")[1]),) + tuple(real[0].shape[1:]), dtype=real[0].dtype) if k.startswith("@zeros:")
+                 else next(it) for k in keys]
+        return torch.cat(parts, dim=0)
+
 
 @torch.no_grad()
 def load_safetensors(model, path: str) -> None:
@@ -112,10 +123,9 @@ def load_safetensors(model, path: str) -> None:
         if fused is not None:                                # the model names its checkpoint tensors itself
             keys = fused.get(name, [name])
             if isinstance(keys[0], (list, tuple)):                   # stacked: one slice per entry (each a concatenation)
-                full = torch.stack([torch.cat([shards.get(k) for k in ks], dim=0) if len(ks) > 1 else shards.get(ks[0])
-                                    for ks in keys])
+                full = torch.stack([shards.cat(ks) for ks in keys])
             else:
-                full = torch.cat([shards.get(k) for k in keys], dim=0) if len(keys) > 1 else shards.get(keys[0])
+                full = shards.cat(keys)
             if tuple(full.shape) != w.full_shape and full.numel() == w.data.numel():
                 full = full.reshape(w.full_shape)                    # scalars stored 0-d, per-head tables stored [H, D]
         elif ".experts.w" in name:

@@ -310,14 +310,17 @@ class GatedAttention(nn.Module):
         assert H % G == 0, "query heads must be a multiple of the key/value heads"
         self.own_kv = spec.kv_from < 0
         Gp = G if self.own_kv else 0
-        self.cols = (H * D, Gp * D, Gp * Dv, H)                     # q | k | v | one output gate per head
+        used = H * D + Gp * D + Gp * Dv + H
+        # q | k | v | one output gate per head | unused rows: the tile kernels read query rows at 16-byte strides
+        self.cols = (H * D, Gp * D, Gp * Dv, H, -used % 8)
         self.qkvg = _matrix(sum(self.cols), width, ctx, dtype, device)
         self.o = _matrix(width, H * Dv, ctx, dtype, device)
         self.q_norm = _param((H * D,), ctx, device)
         self.k_norm = _param((G * D,), ctx, device) if self.own_kv else None
 
     def weights(self, p):
-        yield p + "qkvg", self.qkvg, "normal", [p + "q"] + ([p + "k", p + "v"] if self.own_kv else []) + [p + "g"]
+        pad = [f"@zeros:{self.cols[4]}"] if self.cols[4] else []
+        yield p + "qkvg", self.qkvg, "normal", [p + "q"] + ([p + "k", p + "v"] if self.own_kv else []) + [p + "g"] + pad
         yield p + "o", self.o, "normal", None
         yield p + "q.norm", self.q_norm, "ones", None
         if self.own_kv:
@@ -334,13 +337,13 @@ class GatedAttention(nn.Module):
         s = self.s
         H, G, D, Dv = s.heads, s.kv_heads, s.dim, s.vdim
         T = h.shape[0]
-        nq, nk, nv, ng = self.cols
+        nq, nk, nv, ng, _pad = self.cols
         both = ops.linear(h, self.qkvg.data)
         seqmix.wide_norm_rope_cache(both, self.q_norm.data, self.k_norm.data if self.own_kv else None, self.eps, meta.positions,
                                     None, 1.0, 0, meta.slot_mapping, cache.k, cache.v, H, G if self.own_kv else 0, D, Dv)
         out = torch.zeros(T, H, Dv, dtype=h.dtype, device=h.device)      # padding rows of a captured step stay zero
         seqmix.token_attention(out, both[:, :nq].unflatten(1, (H, D)), None, cache.k, cache.v, meta, G, Dv, s.scale,
-                               gate=both[:, nq + nk + nv:])
+                               gate=both[:, nq + nk + nv:nq + nk + nv + ng])
         return ops.linear(out.view(T, H * Dv), self.o.data)
 
 
@@ -529,7 +532,7 @@ class HyperLayer(nn.Module):
 
     def cache(self, num_blocks, num_slots, dtype, device) -> LayerCache:
         c = self.mixer.cache(num_blocks, num_slots, dtype, device)
-        if self.taps > 1:           # the sequence's last taps-1 mixer inputs, oldest first
+        if self.taps:               # the sequence's last taps-1 mixer inputs, oldest first
             c.shift = torch.zeros(num_slots, self.taps - 1, self.norm1.data.shape[0], dtype=torch.float32, device=device)
         return c
 
