@@ -10,6 +10,8 @@
     python bench.py --sweep                           # SLO frontier: largest offered QPS with ≥ 90 % attainment
     python bench.py --mixers [--sizes small ...]      # side benchmark: Rodelix stacks beside Llama at equal layer sizes
     python bench.py --mixers --models mixtral,vibunex # side benchmark: Vibunex stacks beside Mixtral at equal layer sizes
+    python bench.py --mixers --models mixtral,sevelorn-attention,rodelix-lightning,sevelorn-retention,llama,sevelorn
+                                                      # side benchmark: Sevelorn stacks beside their closest families
 
 One rank per GPU.  ``--tp`` consecutive ranks form one tensor-parallel replica (``dp = gpus / tp`` replicas);
 every replica serves its share (round-robin, the router's stateless policy) of ONE global BurstGPT-like trace

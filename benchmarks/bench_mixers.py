@@ -16,6 +16,13 @@ can be told apart.  Vocabulary 32000 for all.
 squared-ReLU experts) with the closest existing family, a Mixtral stack of the same width, heads and head size: 8 experts,
 2 per token, Mixtral expert width = half the Llama FFN; the Vibunex experts are 1.5× as wide minus 512 with a shared expert
 of 1024 (two matrices instead of three: the same feed-forward FLOPs per token); its recurrence has width / 64 heads of 64.
+
+``--models mixtral,llama,rodelix-lightning,sevelorn,sevelorn-attention,sevelorn-retention`` compares the hyper-connected
+stacks (four fp32 streams, a four-tap input convolution) with their closest families at equal width, heads and head size:
+``sevelorn-attention`` = gated attention (every layer with keys / values of its own) + 8 silu experts, 2 per token, of the
+Mixtral expert width — beside ``mixtral``; ``sevelorn-retention`` = retention (heads of 128 × 128) + a tanh-GELU gated
+feed-forward of the Llama width — beside ``rodelix-lightning`` (mixer) and ``llama`` (feed-forward); ``sevelorn`` = an
+attention layer, an attention layer on the first one's keys / values (both with experts) and a retention layer (dense).
 """
 from __future__ import annotations
 
@@ -62,8 +69,23 @@ def vibunex_raw(width, heads, kv, ffn):
             "layers": [layer] * LAYERS}
 
 
+def sevelorn_raw(width, heads, kv, ffn, kinds):
+    moe = {"kind": "moe", "expert": {"ff": ffn // 2}, "router": {"experts": 8, "top": 2}}
+    dense = {"kind": "dense", "ff": ffn}
+    att = {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 128, "scale": 128 ** -0.5}
+    mk = {
+        "attention": {"type": "attention", "mlp": moe, "mixer": att},
+        "shared_attention": {"type": "attention", "mlp": moe, "mixer": dict(att, kv_from=0)},
+        "retention": {"type": "retention", "mlp": dense,
+                      "mixer": {"heads": heads, "dim": 128, "vdim": 128, "rot": {"base": 1000000.0, "dims": 128},
+                                "decay": [1.0 - 2.0 ** -(3 + 5 * h / heads) for h in range(heads)]}},
+    }
+    return {"architecture": "Sevelorn", "vocab": 32000, "width": width, "streams": 4, "canon": {"taps": 4},
+            "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5}, "layers": [mk[k] for k in kinds]}
+
+
 def model_configs(size):
-    from dli_amd.config import ModelConfig, rodelix_config, vibunex_config
+    from dli_amd.config import ModelConfig, rodelix_config, sevelorn_config, vibunex_config
     s = SIZES[size]
     out = {"llama": ModelConfig(name=f"llama-{size}", arch="llama", vocab_size=32000, hidden_size=s["width"],
                                 intermediate_size=s["ffn"], num_layers=LAYERS, num_heads=s["heads"], num_kv_heads=s["kv"],
@@ -72,6 +94,9 @@ def model_configs(size):
                                  intermediate_size=s["ffn"] // 2, num_layers=LAYERS, num_heads=s["heads"], num_kv_heads=s["kv"],
                                  head_dim=128, max_position=16384, num_experts=8, top_k_experts=2)
     out["vibunex"] = vibunex_config(vibunex_raw(s["width"], s["heads"], s["kv"], s["ffn"]), name=f"vibunex-{size}")
+    for name, kinds in (("sevelorn", ("attention", "shared_attention", "retention")), ("sevelorn-attention", ("attention",) * LAYERS),
+                        ("sevelorn-retention", ("retention",) * LAYERS)):
+        out[name] = sevelorn_config(sevelorn_raw(s["width"], s["heads"], s["kv"], s["ffn"], kinds), name=f"{name}-{size}")
     kinds = ("attention", "lightning", "latent_attention")
     out["rodelix"] = rodelix_config(rodelix_raw(s["width"], s["heads"], s["kv"], s["ffn"], kinds), name=f"rodelix-{size}")
     for k in kinds:

@@ -260,10 +260,11 @@ Tensor dm_relu2_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, c
   TORCH_CHECK(ids.dim() == 2 && ids.size(0) == T && wts.dim() == 2 && wts.size(0) == T && wts.size(1) == ids.size(1), "ids / wts must be [T, K]");
   const int64_t K = ids.size(1);
   Tensor out = at::empty({T, W}, h.options());
-  if (gated && bf && g_dm_grouped_experts && W % 128 == 0 && F % 64 == 0 && E <= 64 && T * K >= 64 && h.is_contiguous() &&
+  if (gated && bf && g_dm_grouped_experts && W % 128 == 0 && F % 64 == 0 && E <= 64 && (T * K >= 64 || F % 128 == 0) && h.is_contiguous() &&
       reinterpret_cast<uintptr_t>(h.data_ptr()) % 16 == 0) {
-    // the grouped GEMMs of the Mixtral path (gate / up tile pairs with the silu product in the first epilogue)
-    moe_experts_forward(h, ids, wts, up, down, K, 0, false, out.data_ptr(), cur_stream(h));
+    // the expert kernels of the Mixtral path: weight streaming at decode size, else grouped GEMMs (gate / up tile pairs with
+    // the silu product in the first epilogue)
+    moe_apply(h, ids, wts, up, down, K, 0, E, 0, out, cur_stream(h));
     return out;
   }
   if (!gated && bf && g_dm_grouped_experts && W % 128 == 0 && F % 128 == 0 && E <= 64 && T * K >= 64 && h.stride(0) % 8 == 0 &&

@@ -370,6 +370,43 @@ void moe_experts_forward(const Tensor& x, const Tensor& ids, const Tensor& wts, 
                       (int)T, (int)H, out, stream);
 }
 
+// ---- experts of tokens whose (expert id, weight) pairs are already on the device: the decode-sized weight-streaming path or
+// the grouped GEMMs, chosen as for the Mixtral block (tile_rows: 0 = by the row count, 128 / 256 = forced)
+void moe_apply(const Tensor& x, const Tensor& ids, const Tensor& wts, const Tensor& w13, const Tensor& w2, int64_t top_k,
+               int64_t expert_offset, int64_t E, int64_t tile_rows, Tensor& out, hipStream_t stream) {
+  const int64_t T = x.size(0), H = x.size(1), El = w13.size(0), I = w13.size(1) / 2;
+  auto i32 = x.options().dtype(at::kInt);
+  const int64_t n = T * top_k;
+  // 256-row tiles when the experts see enough rows to fill them (and the shapes divide): gemm256.hip
+  bool big = n / E >= g_moe_tile256_min_rows;               // expected rows per expert (local or not) under uniform routing
+  if (g_moe_tile_force) big = g_moe_tile_force == 256;
+  if (tile_rows) big = tile_rows == 256;                     // A/B measurements in one process
+  big = big && I % 128 == 0 && H % 256 == 0 && n * std::max(H, I) * 2 < (int64_t(1) << 32) && 2 * I * H * 2 < (int64_t(1) << 32);
+  if (T <= std::min<int64_t>(g_moe_skinny_max_t, 128) && I % 128 == 0 && tile_rows == 0) {
+    // Decode-sized batch: an expert sees ≤ 16 rows (at T ≤ 32 and 2-of-8 routing: nearly always; more rows cost an
+    // extra pass over that expert's weights from cache), so both projections are pure weight streams — the
+    // weight-streaming kernel of skinny_gemm.hip per (expert, 16 weight rows), SwiGLU in between.
+    const int64_t capacity = (n + 127) / 128 * 128 + El * 128, max_tiles = capacity / 128;
+    Tensor sorted = at::empty({capacity}, i32), tile_expert = at::empty({max_tiles}, i32), meta = at::empty({2}, i32);
+    const int64_t tiles = std::min<int64_t>(El, n), rows_pad = (T + 15) / 16 * 16;
+    Tensor gu = at::empty({tiles * rows_pad, 2 * I}, x.options()), act16 = at::empty({tiles * rows_pad, I}, x.options());
+    Tensor y16 = at::empty({n, H}, x.options());
+    dli::launch_moe_align(ids.data_ptr<int>(), (int)n, (int)expert_offset, (int)El, sorted.data_ptr<int>(),
+                          tile_expert.data_ptr<int>(), meta.data_ptr<int>(), (int)capacity, 128, stream);
+    dli::launch_moe_skinny(false, x.data_ptr(), H, w13.data_ptr(), 2 * I * H, sorted.data_ptr<int>(), tile_expert.data_ptr<int>(),
+                           meta.data_ptr<int>(), wts.data_ptr<float>(), (int)top_k, gu.data_ptr(), 2 * I, (int)H, (int)(2 * I),
+                           (int)tiles, (int)T, stream);
+    dli::launch_silu_and_mul(act16.data_ptr(), gu.data_ptr(), (int)(tiles * rows_pad), (int)I, 2 * I, stream);
+    dli::launch_moe_skinny(true, act16.data_ptr(), I, w2.data_ptr(), H * I, sorted.data_ptr<int>(), tile_expert.data_ptr<int>(),
+                           meta.data_ptr<int>(), wts.data_ptr<float>(), (int)top_k, y16.data_ptr(), H, (int)I, (int)H,
+                           (int)tiles, (int)T, stream);
+    dli::launch_moe_sum(y16.data_ptr(), false, 1, n * H, ids.data_ptr<int>(), (int)expert_offset, (int)El, (int)top_k, (int)T,
+                        (int)H, out.data_ptr(), stream);
+    return;
+  }
+  moe_experts_forward(x, ids, wts, w13, w2, top_k, expert_offset, big, out.data_ptr(), stream);
+}
+
 // ---- MoE: route → align → grouped GEMM (SwiGLU epilogue) → grouped GEMM (weighted scatter) → sum ----
 Tensor fused_moe(const Tensor& x, const Tensor& router_logits, const Tensor& w13, const Tensor& w2, int64_t top_k,
                  int64_t expert_offset, int64_t tile_rows, const c10::optional<Tensor>& out_) {
@@ -383,42 +420,11 @@ Tensor fused_moe(const Tensor& x, const Tensor& router_logits, const Tensor& w13
   TORCH_CHECK(router_logits.size(0) == T && w13.size(2) == H && w2.size(0) == El && w2.size(1) == H && w2.size(2) == I);
   TORCH_CHECK(E <= 64 && top_k >= 1 && top_k <= E && H % 128 == 0 && I % 64 == 0, "unsupported MoE shape");
   auto stream = cur_stream(x);
-  auto i32 = x.options().dtype(at::kInt);
   const int64_t n = T * top_k;
-  // 256-row tiles when the experts see enough rows to fill them (and the shapes divide): gemm256.hip
-  bool big = n / E >= g_moe_tile256_min_rows;               // expected rows per expert (local or not) under uniform routing
-  if (g_moe_tile_force) big = g_moe_tile_force == 256;
-  if (tile_rows) big = tile_rows == 256;                     // A/B measurements in one process
-  big = big && I % 128 == 0 && H % 256 == 0 && n * std::max(H, I) * 2 < (int64_t(1) << 32) && 2 * I * H * 2 < (int64_t(1) << 32);
-  const int64_t TR = big ? 256 : 128;
-  const int64_t capacity = (n + TR - 1) / TR * TR + El * TR;
-  const int64_t max_tiles = capacity / TR;
-  Tensor ids = at::empty({n}, i32), wts = at::empty({n}, x.options().dtype(at::kFloat));
-  Tensor sorted = at::empty({capacity}, i32), tile_expert = at::empty({max_tiles}, i32), meta = at::empty({2}, i32);
+  Tensor ids = at::empty({n}, x.options().dtype(at::kInt)), wts = at::empty({n}, x.options().dtype(at::kFloat));
   Tensor out = take_out(out_, T, H, x);
-  if (T <= std::min<int64_t>(g_moe_skinny_max_t, 128) && I % 128 == 0 && tile_rows == 0) {
-    // Decode-sized batch: an expert sees ≤ 16 rows (at T ≤ 32 and 2-of-8 routing: nearly always; more rows cost an
-    // extra pass over that expert's weights from cache), so both projections are pure weight streams — the
-    // weight-streaming kernel of skinny_gemm.hip per (expert, 16 weight rows), SwiGLU in between.
-    const int64_t tiles = std::min<int64_t>(El, n), rows_pad = (T + 15) / 16 * 16;
-    Tensor gu = at::empty({tiles * rows_pad, 2 * I}, x.options()), act16 = at::empty({tiles * rows_pad, I}, x.options());
-    Tensor y16 = at::empty({n, H}, x.options());
-    dli::launch_moe_route(router_logits.data_ptr(), (int)T, (int)E, (int)top_k, ids.data_ptr<int>(), wts.data_ptr<float>(), stream);
-    dli::launch_moe_align(ids.data_ptr<int>(), (int)n, (int)expert_offset, (int)El, sorted.data_ptr<int>(),
-                          tile_expert.data_ptr<int>(), meta.data_ptr<int>(), (int)capacity, 128, stream);
-    dli::launch_moe_skinny(false, x.data_ptr(), H, w13.data_ptr(), 2 * I * H, sorted.data_ptr<int>(), tile_expert.data_ptr<int>(),
-                           meta.data_ptr<int>(), wts.data_ptr<float>(), (int)top_k, gu.data_ptr(), 2 * I, (int)H, (int)(2 * I),
-                           (int)tiles, (int)T, stream);
-    dli::launch_silu_and_mul(act16.data_ptr(), gu.data_ptr(), (int)(tiles * rows_pad), (int)I, 2 * I, stream);
-    dli::launch_moe_skinny(true, act16.data_ptr(), I, w2.data_ptr(), H * I, sorted.data_ptr<int>(), tile_expert.data_ptr<int>(),
-                           meta.data_ptr<int>(), wts.data_ptr<float>(), (int)top_k, y16.data_ptr(), H, (int)I, (int)H,
-                           (int)tiles, (int)T, stream);
-    dli::launch_moe_sum(y16.data_ptr(), false, 1, n * H, ids.data_ptr<int>(), (int)expert_offset, (int)El, (int)top_k, (int)T,
-                        (int)H, out.data_ptr(), stream);
-    return out;
-  }
   dli::launch_moe_route(router_logits.data_ptr(), (int)T, (int)E, (int)top_k, ids.data_ptr<int>(), wts.data_ptr<float>(), stream);
-  moe_experts_forward(x, ids, wts, w13, w2, top_k, expert_offset, big, out.data_ptr(), stream);
+  moe_apply(x, ids, wts, w13, w2, top_k, expert_offset, E, tile_rows, out, stream);
   return out;
 }
 

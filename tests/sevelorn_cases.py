@@ -238,12 +238,14 @@ def case_first_tokens_and_long_decode(tmp, device, dtype):
 # ---------------------------------------------------------------- other sizes
 def other_size_configs():
     big_moe = {"kind": "moe", "expert": {"ff": 64}, "router": {"experts": 6, "top": 3}}
+    wide_moe = {"kind": "moe", "expert": {"ff": 128}, "router": {"experts": 4, "top": 2}}
     return {
         "matrix-core tiles, heads of 64, shared keys, no feed-forward":
             make_cfg([attn(8, 2, 64, 64, 0.15), ret(2, 64, 64, (0.97, 0.999), (32, 1e4)), attn(8, 2, 64, 64, 0.1, kv_from=0)], width=96, vocab=80),
         "matrix-core tiles, heads of 128, one query head per key head":
             make_cfg([attn(2, 2, 128, 128, 0.1), attn(2, 2, 128, 128, 0.1, kv_from=0)], width=64, vocab=70, streams=1, taps=1),
-        "experts as grouped products": make_cfg([attn(2, 1, 64, 64, 0.15, mlp=big_moe), ret(2, 32, 64, (0.9, 0.99), (16, 1e4), mlp=big_moe)],
+        # (an expert width of 128 also takes the weight-streaming kernels at decode size)
+        "experts as grouped products": make_cfg([attn(2, 1, 64, 64, 0.15, mlp=big_moe), ret(2, 32, 64, (0.9, 0.99), (16, 1e4), mlp=wide_moe)],
                                                 width=128, vocab=90, streams=4, taps=2),
         "eight query heads per key head": make_cfg([attn(16, 2, 16, 32, 0.35, mlp=DENSE), attn(8, 1, 32, 16, 0.2)], width=56, vocab=64, streams=5),
         "single heads, every expert chosen, one tap": make_cfg(
