@@ -251,7 +251,7 @@ def other_size_configs():
         "single heads, every expert chosen, one tap": make_cfg(
             [attn(1, 1, 16, 64, 1.0, mlp={"kind": "moe", "expert": {"ff": 8}, "router": {"experts": 7, "top": 7}}),
              ret(1, 40, 8, (0.93,), (2, 1e6), mlp={"kind": "moe", "expert": {"ff": 24}, "router": {"experts": 3, "top": 1}})],
-            width=48, vocab=130, streams=1, taps=1, eps=1e-3, scale=None),
+            width=50, vocab=130, streams=1, taps=1, eps=1e-3, scale=None),      # a width that rules out 16-byte accesses
         "odd head sizes, no rotation, wide state": make_cfg([attn(3, 3, 12, 20, 0.4, mlp=DENSE), ret(2, 100, 70, (0.9, 0.99), None)],
                                                             width=40, vocab=50, streams=3, taps=3),
         "partly rotated heads, seven taps, eight streams": make_cfg([ret(4, 32, 16, (0.5, 0.9, 0.99, 0.999), (6, 50.0)), attn(6, 3, 8, 8, 0.5)],
