@@ -40,9 +40,9 @@ Tensor hm_causal_conv_add(const Tensor& h, const Tensor& w, Tensor state, const 
   TORCH_CHECK(h.dim() == 2, "h must be [T, W]");
   const int64_t T = h.size(0), W = h.size(1);
   check_f32(w, "w");
-  TORCH_CHECK(w.dim() == 2 && w.size(0) == W && w.size(1) >= 1 && w.size(1) <= dli::hm_max_taps(), "w must be [W, taps], taps in 1..",
+  TORCH_CHECK(w.dim() == 2 && w.size(1) == W && w.size(0) >= 1 && w.size(0) <= dli::hm_max_taps(), "w must be [taps, W], taps in 1..",
               dli::hm_max_taps());
-  const int64_t taps = w.size(1);
+  const int64_t taps = w.size(0);
   check_f32(state, "state");
   if (taps > 1)
     TORCH_CHECK(state.dim() == 3 && state.size(1) == taps - 1 && state.size(2) == W, "state must be [slots, taps-1, W]");

@@ -140,7 +140,7 @@ __global__ __launch_bounds__(NT) void stream_mix_norm_kernel(float* __restrict__
 }
 
 // ------------------------------------------------------------------------------------------------ input convolution
-// out[t] = h[t] + Σ_j w[:, j] · h[t - taps + 1 + j] over the rows of the token's own sequence: rows of this step's chunk, the
+// out[t] = h[t] + Σ_j w[j, :] · h[t - taps + 1 + j] (w [taps, W]: a tap's weights are one contiguous row) over the rows of the token's own sequence: rows of this step's chunk, the
 // sequence's state rows (its last taps-1 inputs, oldest first: positions p0-taps+1 … p0-1 for a chunk starting at p0) before
 // the chunk, zero before position 0 (so a reused slot needs no clearing).  One workgroup per token, V columns per thread and trip.
 template <typename O, int V>
@@ -169,14 +169,15 @@ __global__ __launch_bounds__(NT) void causal_conv_add_kernel(const float* __rest
   for (int c = threadIdx.x * V; c < W; c += NT * V) {
     Vec<float, V> a;
     a.load(hr + c);
-    for (int j = 0; j < taps; ++j) {
+#pragma unroll 4
+    for (int j = max(taps - 1 - p, 0); j < taps; ++j) {          // taps that would reach before position 0 are skipped
       const int d = taps - 1 - j;                                 // how far back the tap reaches
-      if (p - d < 0) continue;
       // state row of position p - d: its index counts from the chunk's first position minus (taps - 1)
-      Vec<float, V> v;
+      Vec<float, V> v, wj;
       v.load(d <= back ? hr + c - (int64_t)d * W : st + (int64_t)(taps - 1 - (d - back)) * W + c);
+      wj.load(w + (int64_t)j * W + c);
 #pragma unroll
-      for (int k = 0; k < V; ++k) a.v[k] += w[(c + k) * taps + j] * v.v[k];
+      for (int k = 0; k < V; ++k) a.v[k] += wj.v[k] * v.v[k];
     }
     Vec<O, V> o;
 #pragma unroll
@@ -398,7 +399,7 @@ void launch_hm_causal_conv_add(const float* h, const float* w, int taps, float* 
                                const int* qsl, const int* state_slots, const int* counts, int rows, int seqs, int W, void* out,
                                bool out_bf16, hipStream_t stream) {
   if (rows == 0) return;
-  if (W % 4 == 0 && al16(h) && al16(state) && al16(out))
+  if (W % 4 == 0 && al16(h) && al16(state) && al16(out) && al16(w))
     HM_BF16(out_bf16, O, hipLaunchKernelGGL((causal_conv_add_kernel<O, 4>), dim3(rows), dim3(NT), 0, stream, h, w, taps, state, positions,
                                             token_seq, qsl, state_slots, W, (O*)out));
   else

@@ -505,7 +505,8 @@ class HyperLayer(nn.Module):
         self.links = streams > 0
         S = max(streams, 1)
         self.norm1, self.hc1 = _param((width,), ctx, device), StreamLinks(S, ctx, device)
-        self.conv = _param((width, taps), ctx, device) if taps else None
+        self.conv = _param((width, taps), ctx, device) if taps else None    # as checkpoints store it: a channel's taps together
+        self._conv_taps = None                                               # tap-major copy for the kernel, made at first use
         self.mixer = MIXERS[spec.kind](spec, width, eps, ctx, dtype, device)
         self.ff = None
         if spec.ff:
@@ -546,7 +547,9 @@ class HyperLayer(nn.Module):
         """``x``: fp32 streams ``[T, S, W]``, updated in place; ``h``: this layer's normed mixer input (``read``).  Returns the
         last sublayer's output and its links — the caller's next ``read`` (or the closing norm) writes them back."""
         if self.conv is not None:
-            h = seqmix.causal_conv_add(h, self.conv.data, cache.shift, meta, self.dtype)
+            if self._conv_taps is None:
+                self._conv_taps = self.conv.data.t().contiguous()
+            h = seqmix.causal_conv_add(h, self._conv_taps, cache.shift, meta, self.dtype)
         y = self.mixer(h, meta, cache)
         if self.ff is None:
             return y, self.hc1

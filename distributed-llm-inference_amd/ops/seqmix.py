@@ -554,14 +554,15 @@ def stream_mix_norm(x: torch.Tensor, y: Optional[torch.Tensor], mix: Optional[to
 
 
 def causal_conv_add(h: torch.Tensor, w: torch.Tensor, state: torch.Tensor, meta, out_dtype: torch.dtype) -> torch.Tensor:
-    """``h [T, W]`` fp32; ``w [W, taps]`` fp32.  Row ``t`` of the result is ``h[t] + Σ_j w[:, j] · h[t - taps + 1 + j]`` over the
+    """``h [T, W]`` fp32; ``w [taps, W]`` fp32 (tap-major: the last row weighs the token itself).  Row ``t`` of the result is
+    ``h[t] + Σ_j w[j] · h[t - taps + 1 + j]`` over the
     rows of the same sequence: rows above inside a chunk, the sequence's ``state`` rows ``[slots, taps-1, W]`` (its last
     ``taps-1`` inputs, oldest first) before a chunk's start, zero before position 0.  The state rows are then moved on to
     the sequence's last ``taps-1`` inputs of this step."""
     if h.is_cuda:
         return _hip().hm_causal_conv_add(h, w, state, meta.positions, meta.token_seq, meta.query_start_loc, meta.state_slots,
                                          meta.counts, meta.num_seqs, out_dtype == torch.bfloat16)
-    taps = w.shape[1]
+    taps = w.shape[0]
     out = h.clone()
     for _i, t0, t1, slot in _seq_rows(meta):
         p0 = int(meta.positions[t0])
@@ -572,7 +573,7 @@ def causal_conv_add(h: torch.Tensor, w: torch.Tensor, state: torch.Tensor, meta,
                 hist[r] = 0.0
         ext = torch.cat([hist, h[t0:t1]], dim=0)                                         # [taps-1+n, W]
         for j in range(taps):
-            out[t0:t1] += w[:, j] * ext[j:j + n]
+            out[t0:t1] += w[j] * ext[j:j + n]
         if taps > 1:
             state[slot] = ext[n:]
     return out.to(out_dtype)
