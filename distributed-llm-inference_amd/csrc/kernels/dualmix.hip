@@ -176,6 +176,92 @@ __global__ __launch_bounds__(NT) void wide_norm_rope_cache_kernel(A* __restrict_
     for (int i = threadIdx.x; i < G * Dv; i += NT) v_cache[(int64_t)slot * G * Dv + i] = row[nq + nk + i];
 }
 
+// 4 consecutive row entries ↔ fp32 (16-byte / 8-byte accesses)
+template <typename A> __device__ __forceinline__ f32x4 ldv4(const A* p);
+template <> __device__ __forceinline__ f32x4 ldv4<float>(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+template <> __device__ __forceinline__ f32x4 ldv4<uint16_t>(const uint16_t* p) {
+  const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+  return f32x4{bf2f((uint16_t)v[0]), bf2f((uint16_t)v[1]), bf2f((uint16_t)v[2]), bf2f((uint16_t)v[3])};
+}
+template <typename A> __device__ __forceinline__ void stv4(A* p, f32x4 v);
+template <> __device__ __forceinline__ void stv4<float>(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+template <> __device__ __forceinline__ void stv4<uint16_t>(uint16_t* p, f32x4 v) {
+  bf16x4 o;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = (short)f2bf(v[j]);
+  *reinterpret_cast<bf16x4*>(p) = o;
+}
+
+// The same with four entries per access, for rows whose pieces (q, k, v widths, head size, rotated half) are all multiples of
+// four and 16-byte aligned: a vector of four then never straddles a head or the rotated / unrotated border.
+template <typename A>
+__global__ __launch_bounds__(NT) void wide_norm_rope_cache_v4_kernel(A* __restrict__ qkv, int64_t row_stride, const float* __restrict__ qw,
+                                                                     const float* __restrict__ kw, float eps,
+                                                                     const int* __restrict__ positions, const double* __restrict__ freq,
+                                                                     float mag, int rot_dims, const int* __restrict__ slot_mapping,
+                                                                     A* __restrict__ k_cache, A* __restrict__ v_cache, int H, int G, int D,
+                                                                     int Dv) {
+  extern __shared__ __align__(16) float sh[];
+  __shared__ float red[NT / 64];
+  const int t = blockIdx.x;
+  const int nq = H * D, nk = G * D, half = rot_dims >> 1;
+  float* qs = sh;
+  float* ks = sh + nq;
+  float* cs = ks + nk;
+  float* sn = cs + half;
+  A* row = qkv + (int64_t)t * row_stride;
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x * 4; i < nq; i += NT * 4) {
+    const f32x4 v = ldv4<A>(row + i);
+    *reinterpret_cast<f32x4*>(qs + i) = v;
+    sq += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+  }
+  for (int i = threadIdx.x * 4; i < nk; i += NT * 4) {
+    const f32x4 v = ldv4<A>(row + nq + i);
+    *reinterpret_cast<f32x4*>(ks + i) = v;
+    sk += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+  }
+  if (threadIdx.x < half && freq != nullptr) {
+    const double two_pi = 6.283185307179586476925286766559;
+    double a = (double)positions[t] * freq[threadIdx.x];
+    a -= floor(a / two_pi) * two_pi;
+    cs[threadIdx.x] = cosf((float)a) * mag;
+    sn[threadIdx.x] = sinf((float)a) * mag;
+  }
+  const float iq = 1.f / sqrtf(block_sum<NT>(sq, red) / (float)nq + eps);
+  const float ik = 1.f / sqrtf(block_sum<NT>(sk, red) / (float)max(nk, 1) + eps);
+  for (int i = threadIdx.x * 4; i < nq; i += NT * 4) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(qs + i), w = *reinterpret_cast<const f32x4*>(qw + i);
+    *reinterpret_cast<f32x4*>(qs + i) = f32x4{v[0] * iq * w[0], v[1] * iq * w[1], v[2] * iq * w[2], v[3] * iq * w[3]};
+  }
+  for (int i = threadIdx.x * 4; i < nk; i += NT * 4) {
+    const f32x4 v = *reinterpret_cast<const f32x4*>(ks + i), w = *reinterpret_cast<const f32x4*>(kw + i);
+    *reinterpret_cast<f32x4*>(ks + i) = f32x4{v[0] * ik * w[0], v[1] * ik * w[1], v[2] * ik * w[2], v[3] * ik * w[3]};
+  }
+  __syncthreads();
+  const int slot = slot_mapping[t];
+  for (int i = threadIdx.x * 4; i < nq + nk; i += NT * 4) {
+    const float* src = i < nq ? qs : ks;
+    const int e = i < nq ? i : i - nq;
+    const int d = e % D;
+    f32x4 v = *reinterpret_cast<const f32x4*>(src + e);
+    if (d < half) {
+      const f32x4 o = *reinterpret_cast<const f32x4*>(src + e + half), c = *reinterpret_cast<const f32x4*>(cs + d),
+                  s_ = *reinterpret_cast<const f32x4*>(sn + d);
+      v = f32x4{v[0] * c[0] - o[0] * s_[0], v[1] * c[1] - o[1] * s_[1], v[2] * c[2] - o[2] * s_[2], v[3] * c[3] - o[3] * s_[3]};
+    } else if (d < rot_dims) {
+      const f32x4 o = *reinterpret_cast<const f32x4*>(src + e - half), c = *reinterpret_cast<const f32x4*>(cs + d - half),
+                  s_ = *reinterpret_cast<const f32x4*>(sn + d - half);
+      v = f32x4{v[0] * c[0] + o[0] * s_[0], v[1] * c[1] + o[1] * s_[1], v[2] * c[2] + o[2] * s_[2], v[3] * c[3] + o[3] * s_[3]};
+    }
+    if (i < nq) stv4<A>(row + i, v);
+    else if (slot >= 0) stv4<A>(k_cache + (int64_t)slot * nk + e, v);
+  }
+  if (slot >= 0 && G > 0)
+    for (int i = threadIdx.x * 4; i < G * Dv; i += NT * 4)
+      stv4<A>(v_cache + (int64_t)slot * G * Dv + i, ldv4<A>(row + nq + nk + i));
+}
+
 // ------------------------------------------------------------------------------------------------ attention: sink + mixed heads
 // One workgroup per token; two passes over the sequence's keys in chunks of 64 (a lane per key).  Pass 1: per head the
 // maximum and the denominator (sink included).  Pass 2: normalised weights of all heads for a chunk in LDS, mixed across
@@ -807,8 +893,15 @@ void launch_dm_wide_norm_rope_cache(void* qkv, bool bf16, int64_t row_stride, co
                                     void* k_cache, void* v_cache, int rows, int H, int G, int D, int Dv, hipStream_t stream) {
   if (rows == 0) return;
   const size_t lds = (size_t)(H * D + G * D + rot_dims) * sizeof(float);
-  DM_BF16(bf16, A, hipLaunchKernelGGL(wide_norm_rope_cache_kernel<A>, dim3(rows), dim3(NT), lds, stream, (A*)qkv, row_stride, qw, kw, eps,
-                                      positions, freq, mag, rot_dims, slot_mapping, (A*)k_cache, (A*)v_cache, H, G, D, Dv));
+  auto al = [](const void* p) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool wide = D % 4 == 0 && Dv % 4 == 0 && rot_dims % 8 == 0 && row_stride % 4 == 0 && al(qkv) && al(qw) && al(kw) && al(k_cache) &&
+                    al(v_cache);
+  if (wide)
+    DM_BF16(bf16, A, hipLaunchKernelGGL(wide_norm_rope_cache_v4_kernel<A>, dim3(rows), dim3(NT), lds, stream, (A*)qkv, row_stride, qw, kw,
+                                        eps, positions, freq, mag, rot_dims, slot_mapping, (A*)k_cache, (A*)v_cache, H, G, D, Dv));
+  else
+    DM_BF16(bf16, A, hipLaunchKernelGGL(wide_norm_rope_cache_kernel<A>, dim3(rows), dim3(NT), lds, stream, (A*)qkv, row_stride, qw, kw, eps,
+                                        positions, freq, mag, rot_dims, slot_mapping, (A*)k_cache, (A*)v_cache, H, G, D, Dv));
 }
 
 size_t dm_talk_attention_lds(int H, int D) { return (size_t)(H * D + 2 * H * TA_CHUNK + H * H + 2 * H + TA_CHUNK) * sizeof(float); }

@@ -303,6 +303,7 @@ __global__ __launch_bounds__(NT) void softmax_route_kernel(const A* __restrict__
     float d[TPB];
 #pragma unroll
     for (int k = 0; k < TPB; ++k) d[k] = 0.f;
+#pragma unroll 4
     for (int i = lane * V; i < W; i += 64 * V) {
       Vec<float, V> rw;
       rw.load(router + (int64_t)r * W + i);
