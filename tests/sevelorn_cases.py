@@ -253,7 +253,7 @@ def other_size_configs():
              ret(1, 40, 8, (0.93,), (2, 1e6), mlp={"kind": "moe", "expert": {"ff": 24}, "router": {"experts": 3, "top": 1}})],
             width=50, vocab=130, streams=1, taps=1, eps=1e-3, scale=None),      # a width that rules out 16-byte accesses
         "odd head sizes, no rotation, wide state": make_cfg([attn(3, 3, 12, 20, 0.4, mlp=DENSE), ret(2, 100, 70, (0.9, 0.99), None)],
-                                                            width=40, vocab=50, streams=3, taps=3),
+                                                            width=40, vocab=50, streams=3, taps=6),
         "partly rotated heads, seven taps, eight streams": make_cfg([ret(4, 32, 16, (0.5, 0.9, 0.99, 0.999), (6, 50.0)), attn(6, 3, 8, 8, 0.5)],
                                                                     width=88, vocab=97, streams=8, taps=7, scale=0.5),
     }
