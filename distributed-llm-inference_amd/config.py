@@ -31,7 +31,12 @@ class MixerSpec:
     per head; ``kv_from`` ≥ 0: the layer has no key / value projections and reads that layer's cache) or ``"retention"``
     (linear attention with a per-head decay and no activation or denominator: half-split rotation of the leading
     ``rot_dims`` entries of q and k, keys scaled by ``dim**-0.5``, a ``[D, Dv]`` state per head, per-head unit RMS and a
-    silu gate behind it)."""
+    silu gate behind it), ``"rglru"`` (a gated linear recurrence per channel, ``heads`` blocks of ``dim`` channels: a causal
+    convolution over ``conv_taps`` inputs, block-diagonal recurrence and input gates, decay ``exp(-8 · r · softplus(λ))``,
+    the state multiplied by a tanh-GELU branch) or ``"gated_latent_attention"`` (latent attention whose queries come from a
+    normed latent of size ``q_rank``: half-split rotation with optionally stretched frequencies, sliding ``window``, a
+    per-head ``sink`` in the softmax denominator, an element-wise sigmoid output gate; ``kv_from`` ≥ 0: the layer reads that
+    layer's cached latents and rotated keys and expands them with its own matrices)."""
     kind: str
     heads: int
     dim: int                            # per-head query / key size (latent attention: the unrotated part)
@@ -57,10 +62,17 @@ class MixerSpec:
     kv_from: int = -1                   # gated attention: index of the layer whose cached keys / values this layer reads (-1: its own)
     ff_act: str = "relu2"               # feed-forward activation: "relu2" | "gelu_tanh" (gated dense) | "silu" (gated experts)
     router: str = "sigmoid"             # moe: "sigmoid" (scores, not renormalised) | "softmax" (biased logits, softmax over the chosen)
+                                        # | "softmax_all" (softmax over all logits, a choice bias, renormalised over the chosen)
+    q_rank: int = 0                     # gated latent attention: size of the normed query latent
+    sink: bool = False                  # gated latent attention: a learned per-head logit in the softmax denominator
+    conv_taps: int = 0                  # rglru: taps of the causal convolution in front of the recurrence
+    identity_experts: int = 0           # moe ("softmax_all"): trailing router outputs whose expert returns its input
+    ff_limit: float = 0.0               # moe ("clamped" experts): bound of the gate (above) and of the up projection (both sides)
+    ff_bias: bool = False               # dense feed-forward: the three projections have biases
 
     @property
     def stateful(self) -> bool:
-        return self.kind in ("lightning", "time_mix", "retention") or any(p.stateful for p in self.parts)
+        return self.kind in ("lightning", "time_mix", "retention", "rglru") or any(p.stateful for p in self.parts)
 
     @property
     def cache_row(self) -> tuple:
@@ -70,7 +82,7 @@ class MixerSpec:
             return self.kv_heads * self.dim, self.kv_heads * self.vdim
         if self.kind == "parallel":
             return tuple(sum(w) for w in zip(*(p.cache_row for p in self.parts)))
-        if self.kind == "latent_attention":
+        if self.kind == "latent_attention" or (self.kind == "gated_latent_attention" and self.kv_from < 0):
             return self.kv_rank + self.rot_dim, 0
         return 0, 0
 
@@ -78,6 +90,8 @@ class MixerSpec:
     def state_shape(self) -> tuple:
         if self.kind == "parallel":
             return next((p.state_shape for p in self.parts if p.state_shape), ())
+        if self.kind == "rglru":
+            return (self.heads * self.dim,)
         return (self.heads, self.dim, self.vdim) if self.kind in ("lightning", "time_mix", "retention") else ()
 
 
@@ -117,6 +131,10 @@ class ModelConfig:
     streams: int = 0
     conv_taps: int = 0
     embed_scale: float = 1.0
+    # norm of the hyper-connected layers and the closing norm: "rms_offset" (``u / rms(u) · (1 + w)``) or "layer" (mean taken
+    # off, ``· w``, no bias); ``logit_scale`` multiplies the logits
+    stream_norm: str = "rms_offset"
+    logit_scale: float = 1.0
 
     @property
     def layer_runs(self) -> tuple:
@@ -323,7 +341,63 @@ def sevelorn_config(cfg: dict, name: str = "sevelorn", dtype: str = "bfloat16") 
                        embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)))
 
 
-_CONFIG_READERS = {"Rodelix": rodelix_config, "Vibunex": vibunex_config, "Sevelorn": sevelorn_config}
+def _sinilorn_spec(entry: dict, index: int, layers: list) -> MixerSpec:
+    m, mlp = entry["mixer"], entry.get("mlp")
+    kind = entry["type"]
+    ff = {}
+    if mlp:
+        if mlp.get("kind") == "dense":
+            ff = dict(ff=int(mlp["ff"]), ff_kind="dense", ff_act="silu", ff_bias=True)
+        elif mlp.get("kind") == "moe":
+            r, ex = mlp["router"], mlp["expert"]
+            ff = dict(ff=int(ex["ff"]), ff_kind="moe", ff_act="clamped", ff_limit=float(ex["limit"]), router="softmax_all",
+                      experts=int(r["experts"]), identity_experts=int(r.get("identity") or 0), top=int(r["top"]))
+            if not 1 <= ff["top"] <= ff["experts"] + ff["identity_experts"]:
+                raise ValueError(f"layer {index}: {ff['top']} of {ff['experts']} + {ff['identity_experts']} experts")
+        else:
+            raise ValueError(f"layer {index}: unknown feed-forward kind {mlp.get('kind')!r}")
+    if kind == "rglru":
+        blocks, width = int(m["blocks"]), int(m["width"])
+        if blocks < 1 or width % blocks:
+            raise ValueError(f"layer {index}: {width} channels do not split into {blocks} blocks")
+        return MixerSpec(kind="rglru", heads=blocks, dim=width // blocks, vdim=width // blocks, conv_taps=int(m["conv"]), **ff)
+    if kind == "latent_attention":
+        rot = m.get("rot") or {}
+        sc = rot.get("scaling")
+        src = m.get("kv_from")
+        spec = MixerSpec(kind="gated_latent_attention", heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                         scale=float(m["scale"]), window=int((m.get("mask") or {}).get("size") or 0), kv_rank=int(m["kv_rank"]),
+                         q_rank=int(m["q_rank"]), rot_dim=int(m["rot_dim"]), rot_base=float(rot.get("base", 10000.0)),
+                         rot_dims=int(rot.get("dims", m["rot_dim"])), sink=True, kv_from=-1 if src is None else int(src),
+                         rot_scaling=(float(sc["factor"]), float(sc["original"]), float(sc["fast"]), float(sc["slow"])) if sc else (),
+                         **ff)
+        if spec.rot_dims % 2 or spec.rot_dims > spec.rot_dim:
+            raise ValueError(f"layer {index}: {spec.rot_dims} rotated entries of {spec.rot_dim}")
+        if src is not None:
+            if not 0 <= spec.kv_from < index:
+                raise ValueError(f"layer {index}: latents from layer {src}, which does not run before it")
+            o = layers[spec.kv_from]
+            om = o["mixer"]
+            if o["type"] != "latent_attention" or om.get("kv_from") is not None:
+                raise ValueError(f"layer {index}: layer {src} keeps no latents of its own")
+            if (int(om["kv_rank"]), int(om["rot_dim"])) != (spec.kv_rank, spec.rot_dim):
+                raise ValueError(f"layer {index}: latent sizes differ from those of layer {src}")
+        return spec
+    raise ValueError(f"layer {index}: unknown mixer type {kind!r}")
+
+
+def sinilorn_config(cfg: dict, name: str = "sinilorn", dtype: str = "bfloat16") -> ModelConfig:
+    """``ModelConfig`` of a Sinilorn checkpoint from the dict its ``config.json`` holds."""
+    specs = tuple(_sinilorn_spec(e, i, cfg["layers"]) for i, e in enumerate(cfg["layers"]))
+    att = next((s for s in specs if s.kind == "gated_latent_attention"), specs[0])
+    return ModelConfig(name=name, arch="sinilorn", vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]),
+                       intermediate_size=max([s.ff for s in specs] + [0]), num_layers=len(specs), num_heads=att.heads,
+                       num_kv_heads=1, head_dim=att.dim, max_position=1 << 24, rms_eps=float(cfg["norm"]["eps"]), dtype=dtype,
+                       bos_token_id=0, eos_token_id=-1, layer_specs=specs, streams=int(cfg.get("streams") or 0),
+                       stream_norm="layer", logit_scale=float(cfg.get("logit_scale", 1.0)))
+
+
+_CONFIG_READERS = {"Rodelix": rodelix_config, "Vibunex": vibunex_config, "Sevelorn": sevelorn_config, "Sinilorn": sinilorn_config}
 
 
 def safetensors_shapes(path: str) -> dict:

@@ -298,7 +298,7 @@ Tensor dm_relu2_experts(const Tensor& h, const Tensor& ids, const Tensor& wts, c
   TORCH_CHECK(W * 4 <= kSmMaxLds && K * F * 4 <= kSmMaxLds, "rows too wide");
   Tensor act = at::empty({T * K, F}, h.options());
   dli::launch_dm_experts(h.data_ptr(), bf, h.stride(0), ids.data_ptr<int>(), wts.data_ptr<float>(), (int)K, up.data_ptr(), down.data_ptr(),
-                         (int)T, (int)F, (int)W, act.data_ptr(), out.data_ptr(), gated, cur_stream(h));
+                         (int)T, (int)F, (int)W, act.data_ptr(), out.data_ptr(), gated ? 1 : 0, (int)E, 0.f, cur_stream(h));
   return out;
 }
 

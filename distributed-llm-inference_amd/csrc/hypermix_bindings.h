@@ -6,7 +6,7 @@
 // x [T, S, W] fp32, updated in place when y is given; returns the normed read [T, W] (empty without in_w)
 Tensor hm_stream_mix_norm(Tensor x, const c10::optional<Tensor>& y, const c10::optional<Tensor>& mix, const c10::optional<Tensor>& out_w,
                           const c10::optional<Tensor>& in_w, const c10::optional<Tensor>& norm_w, double eps, double w_offset,
-                          bool out_bf16) {
+                          bool out_bf16, bool center) {
   check_f32(x, "x");
   TORCH_CHECK(x.dim() == 3, "x must be [T, S, W]");
   const int64_t T = x.size(0), S = x.size(1), W = x.size(2);
@@ -30,7 +30,7 @@ Tensor hm_stream_mix_norm(Tensor x, const c10::optional<Tensor>& y, const c10::o
   TORCH_CHECK(W * 4 <= kSmMaxLds, "row too wide");
   Tensor out = at::empty({ip ? T : 0, W}, x.options().dtype(out_bf16 ? at::kBFloat16 : at::kFloat));
   dli::launch_hm_stream_mix_norm(x.data_ptr<float>(), yp, ybf, ys, mp, op, ip, np, (float)eps, (float)w_offset, (int)T, (int)S, (int)W,
-                                 out.data_ptr(), out_bf16, cur_stream(x));
+                                 out.data_ptr(), out_bf16, center, cur_stream(x));
   return out;
 }
 
@@ -87,7 +87,9 @@ Tensor hm_act_mul(const Tensor& x, bool silu) {
   return out;
 }
 
-std::tuple<Tensor, Tensor> hm_softmax_route(const Tensor& h, const Tensor& router, const c10::optional<Tensor>& bias, int64_t K) {
+// all: softmax over all logits, `bias` moves the choice only, weights renormalised over the chosen (rm_softmax_all_route)
+std::tuple<Tensor, Tensor> hm_softmax_route(const Tensor& h, const Tensor& router, const c10::optional<Tensor>& bias, int64_t K,
+                                            bool all) {
   const bool bf = act_bf16(h, "h");
   check_rows(h, "h");
   const int64_t T = h.size(0), W = h.size(1);
@@ -99,6 +101,6 @@ std::tuple<Tensor, Tensor> hm_softmax_route(const Tensor& h, const Tensor& route
   TORCH_CHECK(W * 4 <= kSmMaxLds, "row too wide");
   Tensor ids = at::empty({T, K}, h.options().dtype(at::kInt)), wts = at::empty({T, K}, h.options().dtype(at::kFloat));
   dli::launch_hm_softmax_route(h.data_ptr(), bf, h.stride(0), router.data_ptr<float>(), bp, (int)E, (int)K, (int)T, (int)W,
-                               ids.data_ptr<int>(), wts.data_ptr<float>(), cur_stream(h));
+                               ids.data_ptr<int>(), wts.data_ptr<float>(), all, cur_stream(h));
   return {ids, wts};
 }

@@ -784,23 +784,30 @@ __global__ __launch_bounds__(NT) void sigmoid_route_kernel(const A* __restrict__
 }
 
 // ------------------------------------------------------------------------------------------------ experts, any shape
-// act[p, f] = relu(up[e_p, f, :] · h[t])²  for the routed pair p = t·K + slot; GATED: an expert's rows are F gate rows, then F
-// up rows, and act[p, f] = silu(gate[e_p, f, :] · h[t]) · (up[e_p, f, :] · h[t])
-template <typename A, bool GATED>
+// act[p, f] for the routed pair p = t·K + slot.  ACT 0: relu(up[e_p, f, :] · h[t])².  Gated forms: an expert's rows are F gate
+// rows, then F up rows; with g = gate[e_p, f, :] · h[t] and u = up[e_p, f, :] · h[t], ACT 1: silu(g) · u; ACT 2 (clamped):
+// g' = min(g, limit), u' = clamp(u, ±limit), g' · sigmoid(1.702 g') · (u' + 1).  A pair whose id is not one of the E experts
+// (an identity expert) has no row to compute.
+template <typename A, int ACT>
 __global__ __launch_bounds__(NT) void expert_up_kernel(const A* __restrict__ h, int64_t h_stride, const int* __restrict__ ids, int K,
-                                                       const A* __restrict__ up, int F, int W, A* __restrict__ act) {
+                                                       const A* __restrict__ up, int F, int W, A* __restrict__ act, int E, float limit) {
   extern __shared__ float sh[];
   const int64_t p = blockIdx.x;
   const int64_t t = p / K;
   const int e = ids[p];
+  if (e < 0 || e >= E) return;
   for (int i = threadIdx.x; i < W; i += NT) sh[i] = ldf<A>(h + t * h_stride + i);
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const A* we = up + (int64_t)e * (GATED ? 2 : 1) * F * W;
+  const A* we = up + (int64_t)e * (ACT ? 2 : 1) * F * W;
   for (int f = wave; f < F; f += NT / 64) {
-    if (GATED) {
+    if (ACT == 1) {
       const float g = wave_dot<A>(sh, we + (int64_t)f * W, W), u = wave_dot<A>(sh, we + (int64_t)(F + f) * W, W);
       if (lane == 0) stf<A>(act + p * F + f, g * sigmoid_f(g) * u);
+    } else if (ACT == 2) {
+      const float g = fminf(wave_dot<A>(sh, we + (int64_t)f * W, W), limit);
+      const float u = fminf(fmaxf(wave_dot<A>(sh, we + (int64_t)(F + f) * W, W), -limit), limit);
+      if (lane == 0) stf<A>(act + p * F + f, g * sigmoid_f(1.702f * g) * (u + 1.f));
     } else {
       const float d = fmaxf(wave_dot<A>(sh, we + (int64_t)f * W, W), 0.f);
       if (lane == 0) stf<A>(act + p * F + f, d * d);
@@ -808,20 +815,30 @@ __global__ __launch_bounds__(NT) void expert_up_kernel(const A* __restrict__ h, 
   }
 }
 
-// out[t, c] = Σ_slots wts[t, s] · down[e_s, c, :] · act[t·K + s, :]
+// out[t, c] = Σ_slots wts[t, s] · down[e_s, c, :] · act[t·K + s, :]; a slot whose id is not one of the E experts adds
+// wts[t, s] · hid[t, c] instead (identity expert; hid may be null when every id is an expert's)
 template <typename A>
 __global__ __launch_bounds__(NT) void expert_down_kernel(const A* __restrict__ act, const int* __restrict__ ids, const float* __restrict__ wts,
-                                                         int K, const A* __restrict__ down, int F, int W, A* __restrict__ out) {
+                                                         int K, const A* __restrict__ down, int F, int W, A* __restrict__ out, int E,
+                                                         const A* __restrict__ hid, int64_t hid_stride) {
   extern __shared__ float sh[];
   const int64_t t = blockIdx.x;
-  for (int i = threadIdx.x; i < K * F; i += NT) sh[i] = ldf<A>(act + t * K * F + i);
+  float idw = 0.f;
+  for (int k = 0; k < K; ++k) {
+    const int e = ids[t * K + k];
+    const bool real = e >= 0 && e < E;
+    if (!real && hid != nullptr) idw += wts[t * K + k];
+    for (int i = threadIdx.x; i < F; i += NT) sh[k * F + i] = real ? ldf<A>(act + (t * K + k) * F + i) : 0.f;
+  }
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int c = wave; c < W; c += NT / 64) {
     float s = 0.f;
-    for (int k = 0; k < K; ++k)
-      s += wts[t * K + k] * wave_dot<A>(sh + k * F, down + ((int64_t)ids[t * K + k] * W + c) * F, F);
-    if (lane == 0) stf<A>(out + t * W + c, s);
+    for (int k = 0; k < K; ++k) {
+      const int e = ids[t * K + k];
+      if (e >= 0 && e < E) s += wts[t * K + k] * wave_dot<A>(sh + k * F, down + ((int64_t)e * W + c) * F, F);
+    }
+    if (lane == 0) stf<A>(out + t * W + c, idw != 0.f ? s + idw * ldf<A>(hid + t * hid_stride + c) : s);
   }
 }
 
@@ -1008,17 +1025,21 @@ void launch_dm_sigmoid_route(const void* h, bool bf16, int64_t h_stride, const f
 }
 
 void launch_dm_experts(const void* h, bool bf16, int64_t h_stride, const int* ids, const float* wts, int K, const void* up,
-                       const void* down, int rows, int F, int W, void* act, void* out, bool gated, hipStream_t stream) {
+                       const void* down, int rows, int F, int W, void* act, void* out, int act_kind, int E, float limit,
+                       hipStream_t stream) {
   if (rows == 0) return;
   DM_BF16(bf16, A, {
-    if (gated)
-      hipLaunchKernelGGL((expert_up_kernel<A, true>), dim3(rows * K), dim3(NT), W * sizeof(float), stream, (const A*)h, h_stride, ids, K,
-                         (const A*)up, F, W, (A*)act);
+    if (act_kind == 2)
+      hipLaunchKernelGGL((expert_up_kernel<A, 2>), dim3(rows * K), dim3(NT), W * sizeof(float), stream, (const A*)h, h_stride, ids, K,
+                         (const A*)up, F, W, (A*)act, E, limit);
+    else if (act_kind == 1)
+      hipLaunchKernelGGL((expert_up_kernel<A, 1>), dim3(rows * K), dim3(NT), W * sizeof(float), stream, (const A*)h, h_stride, ids, K,
+                         (const A*)up, F, W, (A*)act, E, limit);
     else
-      hipLaunchKernelGGL((expert_up_kernel<A, false>), dim3(rows * K), dim3(NT), W * sizeof(float), stream, (const A*)h, h_stride, ids, K,
-                         (const A*)up, F, W, (A*)act);
+      hipLaunchKernelGGL((expert_up_kernel<A, 0>), dim3(rows * K), dim3(NT), W * sizeof(float), stream, (const A*)h, h_stride, ids, K,
+                         (const A*)up, F, W, (A*)act, E, limit);
     hipLaunchKernelGGL(expert_down_kernel<A>, dim3(rows), dim3(NT), (size_t)K * F * sizeof(float), stream, (const A*)act, ids, wts, K,
-                       (const A*)down, F, W, (A*)out);
+                       (const A*)down, F, W, (A*)out, E, act_kind == 2 ? (const A*)h : (const A*)nullptr, h_stride);
   });
 }
 

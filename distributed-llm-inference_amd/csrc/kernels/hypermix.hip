@@ -67,12 +67,15 @@ template <typename A, int V> struct Vec {
 // ------------------------------------------------------------------------------------------------ streams: write, read, norm
 // One workgroup per token over x [T, S, W].  With y: x_t ← Σ_s mix[s, t] x_s + out_w[t] · y for all t at once (every column's
 // S values are read before any is written).  With in_w: u = Σ_s in_w[s] x_s of the updated streams is kept in LDS and leaves
-// as u / sqrt(mean(u²) + eps) · (w_offset + norm_w).  MS: compile-time bound of S; a thread takes V columns per trip.
+// as u / sqrt(mean(u²) + eps) · (w_offset + norm_w) — or, with `center`, as the layer norm (u − mean) / sqrt(var + eps) ·
+// (w_offset + norm_w), the variance taken over the deviations in a second pass over the LDS row.  MS: compile-time bound of S;
+// a thread takes V columns per trip.
 template <typename Y, typename O, int MS, int V>
 __global__ __launch_bounds__(NT) void stream_mix_norm_kernel(float* __restrict__ x, const Y* __restrict__ y, int64_t y_stride,
                                                              const float* __restrict__ mix, const float* __restrict__ out_w,
                                                              const float* __restrict__ in_w, const float* __restrict__ norm_w,
-                                                             float eps, float w_offset, int S, int W, O* __restrict__ out) {
+                                                             float eps, float w_offset, int S, int W, O* __restrict__ out,
+                                                             int center) {
   extern __shared__ float us[];
   __shared__ float red[NT / 64];
   __shared__ float cm[MS * MS], co[MS], ci[MS];
@@ -84,7 +87,7 @@ __global__ __launch_bounds__(NT) void stream_mix_norm_kernel(float* __restrict__
   }
   __syncthreads();
   float* xr = x + t * S * W;
-  float sq = 0.f;
+  float sq = 0.f, su = 0.f;
   for (int c = threadIdx.x * V; c < W; c += NT * V) {
     Vec<float, V> xs[MS];
 #pragma unroll
@@ -124,17 +127,29 @@ __global__ __launch_bounds__(NT) void stream_mix_norm_kernel(float* __restrict__
           if (s < S) u += ci[s] * xs[s].v[j];
         us[c + j] = u;
         sq += u * u;
+        su += u;
       }
     }
   }
   if (in_w == nullptr) return;
+  float mean = 0.f;
+  if (center) {                                                   // every thread re-reads the columns it wrote itself
+    mean = block_sum<NT>(su, red) / (float)W;
+    sq = 0.f;
+    for (int c = threadIdx.x * V; c < W; c += NT * V)
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        const float d = us[c + j] - mean;
+        sq += d * d;
+      }
+  }
   const float inv = 1.f / sqrtf(block_sum<NT>(sq, red) / (float)W + eps);
   for (int c = threadIdx.x * V; c < W; c += NT * V) {
     Vec<float, V> nw;
     nw.load(norm_w + c);
     Vec<O, V> o;
 #pragma unroll
-    for (int j = 0; j < V; ++j) o.v[j] = us[c + j] * inv * (w_offset + nw.v[j]);
+    for (int j = 0; j < V; ++j) o.v[j] = (us[c + j] - mean) * inv * (w_offset + nw.v[j]);
     o.store(out + t * W + c);
   }
 }
@@ -281,10 +296,12 @@ __global__ __launch_bounds__(NT) void act_mul_kernel(const A* __restrict__ x, in
 // for all TPB tokens — then wave k picks token k's top-k logits (ties → lowest expert id) and normalises exp(logit − largest)
 // over the picks.  Every pass takes an expert that is still free, whatever the logits hold (a row of padding can carry NaNs;
 // an id outside the experts would index past their weights).  V router entries per lane and trip.
+// `all`: the scores are the softmax over ALL E logits; `bias` is not part of the logits but added to the scores for the choice
+// only, and the weights are the chosen scores divided by their sum (+ 1e-20).
 template <typename A, int TPB, int V>
 __global__ __launch_bounds__(NT) void softmax_route_kernel(const A* __restrict__ h, int64_t h_stride, const float* __restrict__ router,
                                                            const float* __restrict__ bias, int E, int K, int T, int W,
-                                                           int* __restrict__ ids, float* __restrict__ wts) {
+                                                           int* __restrict__ ids, float* __restrict__ wts, int all) {
   extern __shared__ float sh[];                                   // TPB rows of W
   __shared__ float z[TPB][64];
   const int64_t tb = (int64_t)blockIdx.x * TPB;
@@ -312,7 +329,7 @@ __global__ __launch_bounds__(NT) void softmax_route_kernel(const A* __restrict__
 #pragma unroll
         for (int j = 0; j < V; ++j) d[k] += sh[k * W + i + j] * rw.v[j];
     }
-    const float b = bias != nullptr ? bias[r] : 0.f;
+    const float b = bias != nullptr && !all ? bias[r] : 0.f;
 #pragma unroll
     for (int k = 0; k < TPB; ++k) {
       const float s = wave_sum(d[k]);
@@ -328,6 +345,15 @@ __global__ __launch_bounds__(NT) void softmax_route_kernel(const A* __restrict__
       const float v = z[k][lane];
       p = v == v ? v : -INFINITY;
     }
+    float score = 0.f;
+    if (all) {
+      const float mx = wave_max(p);
+      const float ex = (lane < E && mx != -INFINITY) ? expf(p - mx) : 0.f;
+      const float tot = wave_sum(ex);
+      score = tot > 0.f ? ex / tot : 0.f;
+      if (lane < E) p = score + (bias != nullptr ? bias[lane] : 0.f);
+      if (!(p == p)) p = -INFINITY;
+    }
     bool free_lane = lane < E;
     float my_v = -INFINITY, top_v = -INFINITY;
     int my_id = 0;
@@ -341,12 +367,17 @@ __global__ __launch_bounds__(NT) void softmax_route_kernel(const A* __restrict__
         if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
       }
       if (kk == 0) top_v = bv;
-      if (lane == kk) { my_v = bv; my_id = min(bi, E - 1); }
+      const float sv = __shfl(score, min(bi, E - 1) & 63, 64);        // the chosen output's score (softmax over all)
+      if (lane == kk) { my_v = all ? sv : bv; my_id = min(bi, E - 1); }
       if (lane == bi) free_lane = false;
     }
     float e = 0.f;
-    if (lane < K) e = top_v == -INFINITY ? 1.f : expf(my_v - top_v);    // no finite logit at all: equal shares
-    const float sum = wave_sum(e);
+    if (all) {
+      if (lane < K) e = my_v;
+    } else if (lane < K) {
+      e = top_v == -INFINITY ? 1.f : expf(my_v - top_v);                // no finite logit at all: equal shares
+    }
+    const float sum = wave_sum(e) + (all ? 1e-20f : 0.f);
     if (lane < K) {
       ids[t * K + lane] = my_id;
       wts[t * K + lane] = e / sum;
@@ -375,14 +406,14 @@ static bool al16(const void* p) { return p == nullptr || reinterpret_cast<uintpt
 
 void launch_hm_stream_mix_norm(float* x, const void* y, bool y_bf16, int64_t y_stride, const float* mix, const float* out_w,
                                const float* in_w, const float* norm_w, float eps, float w_offset, int rows, int S, int W, void* out,
-                               bool out_bf16, hipStream_t stream) {
+                               bool out_bf16, bool center, hipStream_t stream) {
   if (rows == 0) return;
   const size_t lds = in_w != nullptr ? (size_t)W * sizeof(float) : 0;
   const bool wide = W % 4 == 0 && y_stride % 4 == 0 && al16(x) && al16(y) && al16(norm_w) && al16(out);
 #define HM_SMN(MS, V)                                                                                                               \
   HM_BF16(y_bf16, Y, HM_BF16(out_bf16, O, hipLaunchKernelGGL((stream_mix_norm_kernel<Y, O, MS, V>), dim3(rows), dim3(NT), lds, stream, \
                                                              x, (const Y*)y, y_stride, mix, out_w, in_w, norm_w, eps, w_offset, S, \
-                                                             W, (O*)out)))
+                                                             W, (O*)out, center ? 1 : 0)))
 #define HM_SMN_S(V)            \
   do {                         \
     if (S <= 2) HM_SMN(2, V);  \
@@ -438,7 +469,7 @@ void launch_hm_act_mul(const void* x, bool bf16, int64_t x_stride, int rows, int
 }
 
 void launch_hm_softmax_route(const void* h, bool bf16, int64_t h_stride, const float* router, const float* bias, int E, int K, int rows,
-                             int W, int* ids, float* wts, hipStream_t stream) {
+                             int W, int* ids, float* wts, bool all, hipStream_t stream) {
   if (rows == 0) return;
   const bool wide = W % 4 == 0 && h_stride % 4 == 0 && al16(h) && al16(router);
   // four tokens share a pass over the router rows where their inputs fit the LDS budget together
@@ -446,7 +477,7 @@ void launch_hm_softmax_route(const void* h, bool bf16, int64_t h_stride, const f
 #define HM_ROUTE(TPB, V)                                                                                                      \
   HM_BF16(bf16, A, hipLaunchKernelGGL((softmax_route_kernel<A, TPB, V>), dim3((rows + TPB - 1) / TPB), dim3(NT),              \
                                       (size_t)TPB * W * sizeof(float), stream, (const A*)h, h_stride, router, bias, E, K, rows, W, \
-                                      ids, wts))
+                                      ids, wts, all ? 1 : 0))
   if (four && wide) HM_ROUTE(4, 4);
   else if (four) HM_ROUTE(4, 1);
   else if (wide) HM_ROUTE(1, 4);

@@ -88,14 +88,14 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
                                const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
                                int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* positions,
                                const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
-                               const float* r1, const float* r2, bool bf16, int nsplit, float* part, const void* gate, int64_t g_ts,
+                               const float* r1, const float* r2, bool bf16, int nsplit, float* part, const void* gate, int64_t g_ts, const float* sink,
                                hipStream_t stream);
 int sm_token_attention_splits(int rows, int H, int G);
 bool launch_sm_head_decode_attention(void* out, int64_t o_ts, int64_t o_hs, const void* q1, int64_t q1_ts, int64_t q1_hs, int D1,
                                      const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
                                      int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* positions,
                                      const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
-                                     const float* r1, const float* r2, int nsplit, float* part, const void* gate, int64_t g_ts,
+                                     const float* r1, const float* r2, int nsplit, float* part, const void* gate, int64_t g_ts, const float* sink,
                                      hipStream_t stream);
 int sm_head_decode_splits(int rows, int H, int G);
 bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void* q1, int64_t q1_ts, int64_t q1_hs, int D1,
@@ -103,7 +103,7 @@ bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void*
                               int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* seq_lens,
                               const int* qsl, const int* tile_seq, const int* tile_q0, int num_tiles, const int* counts, int H,
                               int G, float scale, int window, const float* temp, const float* r1, const float* r2,
-                              const void* gate, int64_t g_ts, hipStream_t stream);
+                              const void* gate, int64_t g_ts, const float* sink, hipStream_t stream);
 void launch_sm_lightning_scan(const void* qkvg, bool bf16, int64_t row_stride, float* state, const int* positions, const int* qsl,
                               const int* state_slots, const int* counts, int seqs, int H, int D, int Dv, const float* decay,
                               float* out, int64_t out_part, const int* tile_seq, const int* tile_q0, int num_tiles, float* ws,
@@ -171,12 +171,13 @@ void launch_dm_group_rms_gate(const float* o, int groups, const float* w, float 
 void launch_dm_sigmoid_route(const void* h, bool bf16, int64_t h_stride, const float* router, int router_rows, int E, int K, float scale,
                              int rows, int W, int* ids, float* wts, float* extra, hipStream_t stream);
 void launch_dm_experts(const void* h, bool bf16, int64_t h_stride, const int* ids, const float* wts, int K, const void* up,
-                       const void* down, int rows, int F, int W, void* act, void* out, bool gated, hipStream_t stream);
+                       const void* down, int rows, int F, int W, void* act, void* out, int act_kind, int E, float limit,
+                       hipStream_t stream);     // act_kind 0: relu², 1: silu-gated, 2: clamped gated (ids outside 0..E-1: identity experts)
 
 // hyper-connected stacks (hypermix.hip): several fp32 copies of the stream, input convolution, retention, gated feed-forwards
 void launch_hm_stream_mix_norm(float* x, const void* y, bool y_bf16, int64_t y_stride, const float* mix, const float* out_w,
                                const float* in_w, const float* norm_w, float eps, float w_offset, int rows, int S, int W, void* out,
-                               bool out_bf16, hipStream_t stream);
+                               bool out_bf16, bool center, hipStream_t stream);
 int hm_max_streams();
 int hm_max_taps();
 void launch_hm_causal_conv_add(const float* h, const float* w, int taps, float* state, const int* positions, const int* token_seq,
@@ -186,7 +187,22 @@ void launch_hm_retention_prep(const void* qkvg, bool bf16, int64_t row_stride, c
                               int rows, int H, int D, int Dv, float k_scale, float* out, hipStream_t stream);
 void launch_hm_act_mul(const void* x, bool bf16, int64_t x_stride, int rows, int F, bool silu, void* out, hipStream_t stream);
 void launch_hm_softmax_route(const void* h, bool bf16, int64_t h_stride, const float* router, const float* bias, int E, int K, int rows,
-                             int W, int* ids, float* wts, hipStream_t stream);
+                             int W, int* ids, float* wts, bool all, hipStream_t stream);
+// gated linear recurrences and gated latent attention (recurmix.hip)
+int rm_max_taps();
+void launch_rm_causal_conv(const void* x, bool bf16, int64_t x_stride, const float* w, const float* bias, int taps, float* state,
+                           const int* positions, const int* token_seq, const int* qsl, const int* state_slots, const int* counts,
+                           int rows, int seqs, int C, void* out, bool out_bf16, hipStream_t stream);
+void launch_rm_rglru_scan(const void* z, const void* u, const void* y, bool bf16, int64_t y_stride, const float* gate_bias,
+                          const float* rate, float* state, const int* positions, const int* qsl, const int* state_slots,
+                          const int* counts, int rows, int seqs, int B, int n, void* out, bool out_bf16, hipStream_t stream);
+void launch_rm_latent_norm_cache(const void* proj, bool bf16, int64_t p_stride, int Q, const float* qw, const float* cw, float eps,
+                                 const int* positions, const double* freq, float mag, int rot_dims, const int* slot_mapping, void* cache,
+                                 int rows, int C, int R, void* cq, hipStream_t stream);
+void launch_rm_rotate_heads(void* q, bool bf16, int64_t q_stride, const int* positions, const double* freq, float mag, int rot_dims,
+                            int rows, int H, int D, int R, hipStream_t stream);
+void launch_rm_gate_heads(const void* o, const void* gate, bool bf16, int64_t g_stride, int H, int rows, int Dv, void* out,
+                          hipStream_t stream);
 void launch_dm_relu2_rows(const void* x, bool bf16, int64_t x_stride, int rows, int F, void* out, hipStream_t stream);
 void launch_dm_gated_combine(float* x, float mult, const void* p0, const void* p1, float s0, float s1, const void* g1, int64_t g1_stride,
                              const float* b1, const void* ff, const void* shared, const float* sg, const void* g2, int64_t g2_stride,

@@ -1,0 +1,293 @@
+// Kernels of the stacks that alternate gated linear recurrences with gated latent attention (models/mixers.py:
+// GatedLinearRecurrence, GatedLatentAttention; ops/seqmix.py): the causal per-channel convolution in front of the recurrence
+// with its per-sequence input rows, the recurrence itself (gates, decay, state, output branch), the norms / rotation / cache
+// write of the attention's latents, the rotation of its queries and its element-wise output gate.  (Attention with a sink,
+// the layer norm over several stream copies, score routing and the clamped experts of these stacks are extensions of the
+// kernels in seqmix.hip / hypermix.hip / dualmix.hip.)
+//
+// Arithmetic: convolution sums, gates, decays, the recurrent state, norm statistics and rotation angles (double until
+// reduced) are fp32; activations between GEMMs are the template type float or bf16 (uint16_t bit pattern).
+//
+// Step metadata (int32, static device buffers): positions[T], token_seq[T] (batch row of a token, < 0: padding),
+// query_start_loc[B+1], state_slots[B] (< 0: none), counts[3] = number of valid batch rows.
+#include <algorithm>
+
+#include "common.h"
+#include "kernels.h"
+
+namespace dli {
+
+namespace {
+
+constexpr int NT = 256;
+constexpr int RM_MAX_TAPS = 64;
+
+template <typename A> __device__ __forceinline__ float ldf(const A* p);
+template <> __device__ __forceinline__ float ldf<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ldf<uint16_t>(const uint16_t* p) { return bf2f(*p); }
+template <typename A> __device__ __forceinline__ void stf(A* p, float v);
+template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, float v) { *p = f2bf(v); }
+
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// ------------------------------------------------------------------------------------------------ convolution
+// out[t, c] = bias[c] + Σ_j w[j, c] · x[t - taps + 1 + j, c] over the rows of the token's own sequence: rows of this step's
+// chunk, the sequence's state rows (its last taps-1 inputs, oldest first: positions p0-taps+1 … p0-1 for a chunk starting at
+// p0) before the chunk, nothing before position 0 (so a reused slot needs no clearing).  One workgroup per token; a thread
+// keeps one channel per trip, so all taps of a channel are coalesced row reads.
+template <typename A, typename O>
+__global__ __launch_bounds__(NT) void causal_conv_kernel(const A* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
+                                                         const float* __restrict__ bias, int taps, const float* __restrict__ state,
+                                                         const int* __restrict__ positions, const int* __restrict__ token_seq,
+                                                         const int* __restrict__ qsl, const int* __restrict__ state_slots, int C,
+                                                         O* __restrict__ out) {
+  const int64_t t = blockIdx.x;
+  const int seq = token_seq[t];
+  if (seq < 0 || state_slots[seq] < 0) {                         // padding row
+    for (int c = threadIdx.x; c < C; c += NT) stf<O>(out + t * C + c, 0.f);
+    return;
+  }
+  const int p = positions[t];
+  const int back = (int)t - qsl[seq];                             // rows of the chunk above this one
+  const float* st = state + (int64_t)state_slots[seq] * (taps - 1) * C;
+  const A* xr = x + t * x_stride;
+  for (int c = threadIdx.x; c < C; c += NT) {
+    float a = bias != nullptr ? bias[c] : 0.f;
+    for (int j = max(taps - 1 - p, 0); j < taps; ++j) {           // taps that would reach before position 0 are skipped
+      const int d = taps - 1 - j;                                  // how far back the tap reaches
+      const float v = d <= back ? ldf<A>(xr - (int64_t)d * x_stride + c) : st[(int64_t)(taps - 1 - (d - back)) * C + c];
+      a += w[(int64_t)j * C + c] * v;
+    }
+    stf<O>(out + t * C + c, a);
+  }
+}
+
+// One workgroup per batch row, after the kernel above has read the old rows: the state becomes the sequence's last taps-1
+// inputs.  New row r holds chunk row n-(taps-1)+r when that exists, else old row n+r (written in increasing r by the thread
+// that owns the column, so an old row is read before its turn to be replaced).
+template <typename A>
+__global__ __launch_bounds__(NT) void conv_rows_kernel(const A* __restrict__ x, int64_t x_stride, int taps, float* __restrict__ state,
+                                                       const int* __restrict__ qsl, const int* __restrict__ state_slots,
+                                                       const int* __restrict__ counts, int C) {
+  const int seq = blockIdx.x;
+  if (seq >= counts[3]) return;
+  const int slot = state_slots[seq];
+  const int t0 = qsl[seq], n = qsl[seq + 1] - t0;
+  if (slot < 0 || n <= 0) return;
+  float* st = state + (int64_t)slot * (taps - 1) * C;
+  for (int c = threadIdx.x; c < C; c += NT)
+    for (int r = 0; r < taps - 1; ++r) {
+      const int i = n - (taps - 1) + r;
+      st[(int64_t)r * C + c] = i >= 0 ? ldf<A>(x + (int64_t)(t0 + i) * x_stride + c) : st[(int64_t)(n + r) * C + c];
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ recurrence
+// Per (sequence of the step, channel c = b·n + j), token by token in fp32:
+//   r = sigmoid(z[b, t, j] + gb[c]),  i = sigmoid(z[b, t, n + j] + gb[C + c]),  log a = -rate[c] · r,
+//   S ← exp(log a) · S + sqrt(1 - exp(2 log a)) · i · u[t, c],   out[t, c] = S · gelu_tanh(y[t, c])
+// with S the sequence's state row (zero at position 0), written back after its last token of the step.  A thread owns one
+// channel of one sequence; the next token's operands are fetched while the current one is applied.
+template <typename A, typename O>
+__global__ __launch_bounds__(NT) void rglru_scan_kernel(const A* __restrict__ z, const A* __restrict__ u, const A* __restrict__ y,
+                                                        int64_t y_stride, const float* __restrict__ gb, const float* __restrict__ rate,
+                                                        float* __restrict__ state, const int* __restrict__ positions,
+                                                        const int* __restrict__ qsl, const int* __restrict__ state_slots,
+                                                        const int* __restrict__ counts, int T, int B, int n, O* __restrict__ out) {
+  const int seq = blockIdx.y;
+  if (seq >= counts[3]) return;
+  const int slot = state_slots[seq];
+  const int t0 = qsl[seq], t1 = qsl[seq + 1];
+  if (slot < 0 || t1 <= t0) return;
+  const int C = B * n;
+  const int c = blockIdx.x * NT + threadIdx.x;
+  if (c >= C) return;
+  const int b = c / n, j = c - b * n;
+  const float br = gb[c], bi = gb[C + c], rt = rate[c];
+  float* sp = state + (int64_t)slot * C + c;
+  float S = positions[t0] > 0 ? *sp : 0.f;
+  const A* zp = z + ((int64_t)b * T + t0) * 2 * n + j;
+  float zr = ldf<A>(zp), zi = ldf<A>(zp + n), uu = ldf<A>(u + (int64_t)t0 * C + c), yy = ldf<A>(y + (int64_t)t0 * y_stride + c);
+  for (int t = t0; t < t1; ++t) {
+    const float czr = zr, czi = zi, cu = uu, cy = yy;
+    if (t + 1 < t1) {
+      zp += 2 * n;
+      zr = ldf<A>(zp);
+      zi = ldf<A>(zp + n);
+      uu = ldf<A>(u + (int64_t)(t + 1) * C + c);
+      yy = ldf<A>(y + (int64_t)(t + 1) * y_stride + c);
+    }
+    const float la = -rt * sigmoid_f(czr + br);
+    const float a = expf(la);
+    S = a * S + sqrtf(-expm1f(2.f * la)) * sigmoid_f(czi + bi) * cu;
+    stf<O>(out + (int64_t)t * C + c, S * gelu_tanh_f(cy));
+  }
+  *sp = S;
+}
+
+// ------------------------------------------------------------------------------------------------ latents: norms, rotation, cache
+// One workgroup per token.  proj row = [query latent (Q) | key / value latent (C) | shared key part (R) | …]: the query latent
+// leaves as cq[t] = v / sqrt(mean(v²) + eps) · qw; with a cache, the key / value latent (normed the same way with cw) and the
+// key part — entries i and i + rot_dims/2 turned by position · freq[i], cosine and sine times mag — go to the cache row
+// slot_mapping[t] (< 0: none).
+template <typename A>
+__global__ __launch_bounds__(NT) void latent_norm_cache_kernel(const A* __restrict__ proj, int64_t p_stride, int Q,
+                                                               const float* __restrict__ qw, const float* __restrict__ cw, float eps,
+                                                               const int* __restrict__ positions, const double* __restrict__ freq,
+                                                               float mag, int rot_dims, const int* __restrict__ slot_mapping,
+                                                               A* __restrict__ cache, int C, int R, A* __restrict__ cq) {
+  extern __shared__ float sh[];          // cos[rot_dims/2], sin[rot_dims/2]
+  __shared__ float red[NT / 64];
+  const int64_t t = blockIdx.x;
+  const int half = rot_dims >> 1;
+  const A* row = proj + t * p_stride;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < Q; i += NT) {
+    const float v = ldf<A>(row + i);
+    ss += v * v;
+  }
+  const float qinv = 1.f / sqrtf(block_sum<NT>(ss, red) / (float)Q + eps);
+  for (int i = threadIdx.x; i < Q; i += NT) stf<A>(cq + t * Q + i, ldf<A>(row + i) * qinv * qw[i]);
+  if (cache == nullptr) return;
+  const int slot = slot_mapping[t];
+  if (slot < 0) return;                                             // whole workgroup
+  const double pos = (double)positions[t];
+  for (int i = threadIdx.x; i < half; i += NT) {
+    double a = pos * freq[i];
+    a -= 6.283185307179586476925 * floor(a * 0.15915494309189533577);    // reduced in double, then exact enough in fp32
+    double sn, cs;
+    sincos(a, &sn, &cs);
+    sh[i] = (float)cs * mag;
+    sh[half + i] = (float)sn * mag;
+  }
+  const A* crow = row + Q;
+  ss = 0.f;
+  for (int i = threadIdx.x; i < C; i += NT) {
+    const float v = ldf<A>(crow + i);
+    ss += v * v;
+  }
+  const float inv = 1.f / sqrtf(block_sum<NT>(ss, red) / (float)C + eps);      // (block_sum's barriers also publish sh)
+  A* dst = cache + (int64_t)slot * (C + R);
+  for (int i = threadIdx.x; i < C; i += NT) stf<A>(dst + i, ldf<A>(crow + i) * inv * cw[i]);
+  for (int i = threadIdx.x; i < R; i += NT) {
+    float v = ldf<A>(crow + C + i);
+    if (i < half) {
+      const float o = ldf<A>(crow + C + i + half);
+      v = v * sh[i] - o * sh[half + i];
+    } else if (i < rot_dims) {
+      const float o = ldf<A>(crow + C + i - half);
+      v = v * sh[i - half] + o * sh[i];
+    }
+    stf<A>(dst + C + i, v);
+  }
+}
+
+// In place on q [T, H·(D+R)]: entries D+i and D+i+rot_dims/2 of every head turned by position · freq[i], cosine and sine
+// times mag.  One workgroup per token, a thread per pair and trip (both entries read before either is written).
+template <typename A>
+__global__ __launch_bounds__(NT) void rotate_heads_kernel(A* __restrict__ q, int64_t q_stride, const int* __restrict__ positions,
+                                                          const double* __restrict__ freq, float mag, int rot_dims, int H, int D, int R) {
+  extern __shared__ float sh[];
+  const int64_t t = blockIdx.x;
+  const int half = rot_dims >> 1;
+  const double pos = (double)positions[t];
+  for (int i = threadIdx.x; i < half; i += NT) {
+    double a = pos * freq[i];
+    a -= 6.283185307179586476925 * floor(a * 0.15915494309189533577);
+    double sn, cs;
+    sincos(a, &sn, &cs);
+    sh[i] = (float)cs * mag;
+    sh[half + i] = (float)sn * mag;
+  }
+  __syncthreads();
+  A* row = q + t * q_stride;
+  for (int idx = threadIdx.x; idx < H * half; idx += NT) {
+    const int h = idx / half, i = idx - h * half;
+    A* p = row + (int64_t)h * (D + R) + D + i;
+    const float a = ldf<A>(p), b = ldf<A>(p + half);
+    stf<A>(p, a * sh[i] - b * sh[half + i]);
+    stf<A>(p + half, b * sh[i] + a * sh[half + i]);
+  }
+}
+
+// out[t, h·Dv + d] = o[h, t, d] · sigmoid(gate[t, h·Dv + d])
+template <typename A>
+__global__ __launch_bounds__(NT) void gate_heads_kernel(const A* __restrict__ o, const A* __restrict__ gate, int64_t g_stride, int H,
+                                                        int T, int Dv, A* __restrict__ out) {
+  const int64_t n = (int64_t)T * H * Dv;
+  for (int64_t i = (int64_t)blockIdx.x * NT + threadIdx.x; i < n; i += (int64_t)gridDim.x * NT) {
+    const int64_t t = i / (H * Dv);
+    const int r = (int)(i - t * (H * Dv));
+    const int h = r / Dv, d = r - h * Dv;
+    stf<A>(out + i, ldf<A>(o + ((int64_t)h * T + t) * Dv + d) * sigmoid_f(ldf<A>(gate + t * g_stride + r)));
+  }
+}
+
+}  // namespace
+
+// ================================================================================================ launchers
+#define RM_BF16(flag, T, ...) \
+  do {                        \
+    if (flag) {               \
+      using T = uint16_t;     \
+      __VA_ARGS__;            \
+    } else {                  \
+      using T = float;        \
+      __VA_ARGS__;            \
+    }                         \
+  } while (0)
+
+int rm_max_taps() { return RM_MAX_TAPS; }
+
+void launch_rm_causal_conv(const void* x, bool bf16, int64_t x_stride, const float* w, const float* bias, int taps, float* state,
+                           const int* positions, const int* token_seq, const int* qsl, const int* state_slots, const int* counts,
+                           int rows, int seqs, int C, void* out, bool out_bf16, hipStream_t stream) {
+  if (rows == 0) return;
+  RM_BF16(bf16, A, RM_BF16(out_bf16, O, hipLaunchKernelGGL((causal_conv_kernel<A, O>), dim3(rows), dim3(NT), 0, stream, (const A*)x,
+                                                           x_stride, w, bias, taps, state, positions, token_seq, qsl, state_slots, C,
+                                                           (O*)out)));
+  if (taps > 1 && seqs > 0)
+    RM_BF16(bf16, A, hipLaunchKernelGGL(conv_rows_kernel<A>, dim3(seqs), dim3(NT), 0, stream, (const A*)x, x_stride, taps, state, qsl,
+                                        state_slots, counts, C));
+}
+
+void launch_rm_rglru_scan(const void* z, const void* u, const void* y, bool bf16, int64_t y_stride, const float* gate_bias,
+                          const float* rate, float* state, const int* positions, const int* qsl, const int* state_slots,
+                          const int* counts, int rows, int seqs, int B, int n, void* out, bool out_bf16, hipStream_t stream) {
+  if (rows == 0 || seqs == 0) return;
+  const dim3 grid((B * n + NT - 1) / NT, seqs);
+  RM_BF16(bf16, A, RM_BF16(out_bf16, O, hipLaunchKernelGGL((rglru_scan_kernel<A, O>), grid, dim3(NT), 0, stream, (const A*)z, (const A*)u,
+                                                           (const A*)y, y_stride, gate_bias, rate, state, positions, qsl, state_slots,
+                                                           counts, rows, B, n, (O*)out)));
+}
+
+void launch_rm_latent_norm_cache(const void* proj, bool bf16, int64_t p_stride, int Q, const float* qw, const float* cw, float eps,
+                                 const int* positions, const double* freq, float mag, int rot_dims, const int* slot_mapping, void* cache,
+                                 int rows, int C, int R, void* cq, hipStream_t stream) {
+  if (rows == 0) return;
+  RM_BF16(bf16, A, hipLaunchKernelGGL(latent_norm_cache_kernel<A>, dim3(rows), dim3(NT), std::max(rot_dims, 2) * sizeof(float), stream,
+                                      (const A*)proj, p_stride, Q, qw, cw, eps, positions, freq, mag, rot_dims, slot_mapping, (A*)cache,
+                                      C, R, (A*)cq));
+}
+
+void launch_rm_rotate_heads(void* q, bool bf16, int64_t q_stride, const int* positions, const double* freq, float mag, int rot_dims,
+                            int rows, int H, int D, int R, hipStream_t stream) {
+  if (rows == 0 || rot_dims == 0) return;
+  RM_BF16(bf16, A, hipLaunchKernelGGL(rotate_heads_kernel<A>, dim3(rows), dim3(NT), rot_dims * sizeof(float), stream, (A*)q, q_stride,
+                                      positions, freq, mag, rot_dims, H, D, R));
+}
+
+void launch_rm_gate_heads(const void* o, const void* gate, bool bf16, int64_t g_stride, int H, int rows, int Dv, void* out,
+                          hipStream_t stream) {
+  const int64_t n = (int64_t)rows * H * Dv;
+  if (n == 0) return;
+  const int blocks = (int)std::min<int64_t>((n + NT - 1) / NT, 16384);
+  RM_BF16(bf16, A, hipLaunchKernelGGL(gate_heads_kernel<A>, dim3(blocks), dim3(NT), 0, stream, (const A*)o, (const A*)gate, g_stride, H,
+                                      rows, Dv, (A*)out));
+}
+
+}  // namespace dli

@@ -498,7 +498,7 @@ __global__ __launch_bounds__(NT) void token_attention_kernel(
     const A* __restrict__ vc, int rowv, int vhead, int Dv, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ token_seq, int H, int G, float scale, int window,
     const float* __restrict__ temp, const float* __restrict__ r1, const float* __restrict__ r2, int nsplit,
-    float* __restrict__ part, const A* __restrict__ gate, int64_t g_ts) {
+    float* __restrict__ part, const A* __restrict__ gate, int64_t g_ts, const float* __restrict__ sink) {
   extern __shared__ float sh[];          // q [HG][Dk] | acc [4 waves][HG][Dv] | m [4][HG] | l [4][HG]
   constexpr int NW = NT / 64;
   const int64_t t = blockIdx.x;
@@ -673,6 +673,7 @@ __global__ __launch_bounds__(NT) void token_attention_kernel(
     }
     if (nsplit == 1) {
       const float gm = gate != nullptr ? 1.f / (1.f + expf(-ldf<A>(gate + t * g_ts + h0 + hh))) : 1.f;
+      if (sink != nullptr) L += expf(sink[h0 + hh] - M);            // a logit without key or value in the denominator
       stf<A>(out + t * o_ts + (h0 + hh) * o_hs + e, o / L * gm);
     } else {
       float* pr = part + ((t * H + (h0 + hh)) * nsplit + blockIdx.z) * (int64_t)(Dv + 2);
@@ -690,7 +691,7 @@ template <typename A>
 __global__ __launch_bounds__(128) void token_attention_merge_kernel(A* __restrict__ out, int64_t o_ts, int64_t o_hs,
                                                                     const float* __restrict__ part,
                                                                     const int* __restrict__ token_seq, int H, int Dv,
-                                                                    int nsplit, const A* __restrict__ gate, int64_t g_ts) {
+                                                                    int nsplit, const A* __restrict__ gate, int64_t g_ts, const float* __restrict__ sink) {
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y;
   if (token_seq[t] < 0) return;
@@ -705,6 +706,7 @@ __global__ __launch_bounds__(128) void token_attention_merge_kernel(A* __restric
     f[z] = mz == -INFINITY ? 0.f : expf(mz - M);
     if (z < nsplit) L += f[z] * pr[z * (Dv + 2) + 1];
   }
+  if (sink != nullptr) L += expf(sink[h] - M);
   const float rl = (gate != nullptr ? 1.f / (1.f + expf(-ldf<A>(gate + t * g_ts + h))) : 1.f) / L;
   for (int e = threadIdx.x; e < Dv; e += 128) {
     float o = 0.f;
@@ -732,7 +734,7 @@ __global__ __launch_bounds__(NT * HW) void tile_attention_kernel(
     const int* __restrict__ seq_lens, const int* __restrict__ qsl, const int* __restrict__ tile_seq,
     const int* __restrict__ tile_q0, int num_tiles, const int* __restrict__ counts, int H, int G, float scale, int window,
     const float* __restrict__ temp, const float* __restrict__ r1, const float* __restrict__ r2,
-    const uint16_t* __restrict__ gate, int64_t g_ts) {
+    const uint16_t* __restrict__ gate, int64_t g_ts, const float* __restrict__ sink) {
   extern __shared__ __align__(16) uint16_t tl[];
   const int ntiles = counts != nullptr ? min(counts[2], num_tiles) : num_tiles;
   // the host walks causal tiles longest-first from the END of the list
@@ -872,6 +874,7 @@ __global__ __launch_bounds__(NT * HW) void tile_attention_kernel(
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!qvalid) return;
+  if (sink != nullptr) l += fast_exp2(sink[h] * 1.4426950408889634f - m);
   const float rl = (gate != nullptr ? 1.f / (1.f + expf(-bf2f(gate[tq * g_ts + h]))) : 1.f) / l;
   uint16_t* orow = out + tq * o_ts + h * o_hs;
 #pragma unroll
@@ -899,7 +902,7 @@ __global__ __launch_bounds__(NT) void head_decode_attention_kernel(
     const uint16_t* __restrict__ vc, int rowv, int vhead, int Dv, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ positions, const int* __restrict__ token_seq, int H, int G, int groups, float scale, int window,
     const float* __restrict__ temp, const float* __restrict__ r1, const float* __restrict__ r2, int nsplit,
-    float* __restrict__ part, const uint16_t* __restrict__ gate, int64_t g_ts) {
+    float* __restrict__ part, const uint16_t* __restrict__ gate, int64_t g_ts, const float* __restrict__ sink) {
   extern __shared__ __align__(16) uint16_t tl[];
   const int64_t t = blockIdx.x;
   const int seq = token_seq[t];
@@ -1019,6 +1022,7 @@ __global__ __launch_bounds__(NT) void head_decode_attention_kernel(
   l += __shfl_xor(l, 32, 64);
   if (!hvalid) return;
   if (nsplit == 1) {
+    if (sink != nullptr) l += fast_exp2(sink[h] * 1.4426950408889634f - m);
     const float rl = (gate != nullptr ? 1.f / (1.f + expf(-bf2f(gate[t * g_ts + h]))) : 1.f) / l;
     uint16_t* orow = out + t * o_ts + h * o_hs;
 #pragma unroll
@@ -1275,11 +1279,11 @@ static void token_attention_hg(int hg, dim3 grid, size_t lds, hipStream_t stream
                                int64_t q1_ts, int64_t q1_hs, int D1, const A* q2, int64_t q2_ts, int64_t q2_hs, int D2, const A* kc,
                                int rowk, const A* vc, int rowv, int vhead, int Dv, const int* bt, int max_blocks, const int* pos,
                                const int* tseq, int H, int G, float scale, int window, const float* temp, const float* r1,
-                               const float* r2, int nsplit, float* part, const A* gate, int64_t g_ts) {
+                               const float* r2, int nsplit, float* part, const A* gate, int64_t g_ts, const float* __restrict__ sink) {
 #define SM_ATT(HGV)                                                                                                              \
   hipLaunchKernelGGL((token_attention_kernel<A, VPL, HGV>), grid, dim3(NT), lds, stream, out, o_ts, o_hs, q1, q1_ts, q1_hs, D1,  \
                      q2, q2_ts, q2_hs, D2, kc, rowk, vc, rowv, vhead, Dv, bt, max_blocks, pos, tseq, H, G, scale, window, temp,  \
-                     r1, r2, nsplit, part, gate, g_ts)
+                     r1, r2, nsplit, part, gate, g_ts, sink)
   if (hg == 1) SM_ATT(1);
   else if (hg == 2) SM_ATT(2);
   else SM_ATT(4);
@@ -1290,7 +1294,7 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
                                const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
                                int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* positions,
                                const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
-                               const float* r1, const float* r2, bool bf16, int nsplit, float* part, const void* gate, int64_t g_ts,
+                               const float* r1, const float* r2, bool bf16, int nsplit, float* part, const void* gate, int64_t g_ts, const float* sink,
                                hipStream_t stream) {
   if (rows == 0) return;
   if (Dv > 512) {
@@ -1299,7 +1303,7 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
       launch_sm_token_attention(bf16 ? (void*)((uint16_t*)out + e) : (void*)((float*)out + e), o_ts, o_hs, q1, q1_ts, q1_hs, D1, q2,
                                 q2_ts, q2_hs, D2, kc, rowk, bf16 ? (const void*)((const uint16_t*)vc + e) : (const void*)((const float*)vc + e),
                                 rowv, vhead, std::min(512, Dv - e), block_tables, max_blocks, positions, token_seq, rows, H, G, scale,
-                                window, temp, r1, r2, bf16, 1, nullptr, gate, g_ts, stream);
+                                window, temp, r1, r2, bf16, 1, nullptr, gate, g_ts, sink, stream);
     return;
   }
   // heads per workgroup: as many of the heads sharing a key / value head as divide their number and fit the LDS budget
@@ -1314,7 +1318,7 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
   SM_DISPATCH_BF16(bf16, A, (token_attention_hg<A, VPLV>(hg, grid, lds, stream, (A*)out, o_ts, o_hs, (const A*)q1, q1_ts, q1_hs, \
                                                          D1, (const A*)q2, q2_ts, q2_hs, D2, (const A*)kc, rowk, (const A*)vc,   \
                                                          rowv, vhead, Dv, block_tables, max_blocks, positions, token_seq, H, G,  \
-                                                         scale, window, temp, r1, r2, nsplit, part, (const A*)gate, g_ts)))
+                                                         scale, window, temp, r1, r2, nsplit, part, (const A*)gate, g_ts, sink)))
   if (nv <= 1) SM_ATT_V(1);
   else if (nv <= 2) SM_ATT_V(2);
   else if (nv <= 4) SM_ATT_V(4);
@@ -1322,7 +1326,7 @@ void launch_sm_token_attention(void* out, int64_t o_ts, int64_t o_hs, const void
 #undef SM_ATT_V
   if (nsplit > 1)
     SM_DISPATCH_BF16(bf16, A, hipLaunchKernelGGL(token_attention_merge_kernel<A>, dim3(rows, H), dim3(128), 0, stream, (A*)out, o_ts,
-                                                 o_hs, (const float*)part, token_seq, H, Dv, nsplit, (const A*)gate, g_ts));
+                                                 o_hs, (const float*)part, token_seq, H, Dv, nsplit, (const A*)gate, g_ts, sink));
 }
 
 // workgroups of a per-token attention launch over `rows` tokens: long key ranges are cut so that about 1024 exist
@@ -1340,7 +1344,7 @@ bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void*
                               int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* seq_lens,
                               const int* qsl, const int* tile_seq, const int* tile_q0, int num_tiles, const int* counts, int H,
                               int G, float scale, int window, const float* temp, const float* r1, const float* r2,
-                              const void* gate, int64_t g_ts, hipStream_t stream) {
+                              const void* gate, int64_t g_ts, const float* sink, hipStream_t stream) {
   const int Dk = D1 + D2, KS = (Dk + 31) / 32, MT = Dv / 16;
   auto al = [](const void* p, int64_t a) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % a == 0; };
   const bool ok = D1 % 8 == 0 && D2 % 8 == 0 && Dv % 16 == 0 && KS <= 18 && MT <= 32 && rowk % 8 == 0 && rowv % 8 == 0 &&
@@ -1363,7 +1367,7 @@ bool launch_sm_tile_attention(void* out, int64_t o_ts, int64_t o_hs, const void*
     hipLaunchKernelGGL((tile_attention_kernel<KSM, MTM, HWV>), grid, dim3(NT * HWV), lds, stream, (uint16_t*)out, o_ts, o_hs,    \
                        (const uint16_t*)q1, q1_ts, q1_hs, D1, (const uint16_t*)q2, q2_ts, q2_hs, D2, (const uint16_t*)kc, rowk,  \
                        (const uint16_t*)vc, rowv, vhead, Dv, block_tables, max_blocks, seq_lens, qsl, tile_seq, tile_q0,        \
-                       num_tiles, counts, H, G, scale, window, temp, r1, r2, (const uint16_t*)gate, g_ts);                       \
+                       num_tiles, counts, H, G, scale, window, temp, r1, r2, (const uint16_t*)gate, g_ts, sink);                       \
   } while (0)
 #define SM_TILE(KSM, MTM)              \
   do {                                 \
@@ -1383,7 +1387,7 @@ bool launch_sm_head_decode_attention(void* out, int64_t o_ts, int64_t o_hs, cons
                                      const void* q2, int64_t q2_ts, int64_t q2_hs, int D2, const void* kc, int rowk, const void* vc,
                                      int rowv, int vhead, int Dv, const int* block_tables, int max_blocks, const int* positions,
                                      const int* token_seq, int rows, int H, int G, float scale, int window, const float* temp,
-                                     const float* r1, const float* r2, int nsplit, float* part, const void* gate, int64_t g_ts,
+                                     const float* r1, const float* r2, int nsplit, float* part, const void* gate, int64_t g_ts, const float* sink,
                                      hipStream_t stream) {
   const int Dk = D1 + D2, KS = (Dk + 31) / 32, MT = Dv / 16, per = H / G;
   auto al = [](const void* p, int64_t a) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % a == 0; };
@@ -1406,7 +1410,7 @@ bool launch_sm_head_decode_attention(void* out, int64_t o_ts, int64_t o_hs, cons
     hipLaunchKernelGGL((head_decode_attention_kernel<KSM, MTQV>), grid, dim3(NT), lds, stream, (uint16_t*)out, o_ts, o_hs,       \
                        (const uint16_t*)q1, q1_ts, q1_hs, D1, (const uint16_t*)q2, q2_ts, q2_hs, D2, (const uint16_t*)kc, rowk,  \
                        (const uint16_t*)vc, rowv, vhead, Dv, block_tables, max_blocks, positions, token_seq, H, G, groups, scale,\
-                       window, temp, r1, r2, nsplit, part, (const uint16_t*)gate, g_ts);                                         \
+                       window, temp, r1, r2, nsplit, part, (const uint16_t*)gate, g_ts, sink);                                         \
   } while (0)
   if (KS <= 4 && MT <= 8) SM_HD(4, 2);
   else if (KS <= 8 && MT <= 16) SM_HD(8, 4);
@@ -1414,7 +1418,7 @@ bool launch_sm_head_decode_attention(void* out, int64_t o_ts, int64_t o_hs, cons
 #undef SM_HD
   if (nsplit > 1)
     hipLaunchKernelGGL(token_attention_merge_kernel<uint16_t>, dim3(rows, H), dim3(128), 0, stream, (uint16_t*)out, o_ts, o_hs,
-                       (const float*)part, token_seq, H, Dv, nsplit, (const uint16_t*)gate, g_ts);
+                       (const float*)part, token_seq, H, Dv, nsplit, (const uint16_t*)gate, g_ts, sink);
   return true;
 }
 

@@ -181,7 +181,7 @@ void sm_token_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor
                         const c10::optional<Tensor>& v_cache, const Tensor& block_tables, const Tensor& positions,
                         const Tensor& token_seq, int64_t G, int64_t Dv, double scale, int64_t window, const c10::optional<Tensor>& temp,
                         const c10::optional<Tensor>& r1, const c10::optional<Tensor>& r2, int64_t rows,
-                        const c10::optional<Tensor>& gate) {
+                        const c10::optional<Tensor>& gate, const c10::optional<Tensor>& sink) {
   const bool bf = act_bf16(q1, "q1");
   TORCH_CHECK(q1.dim() == 3 && q1.stride(2) == 1, "q1 must be [T, H, D1] with a contiguous last dim");
   TORCH_CHECK(rows < 0 || rows <= q1.size(0), "rows past the batch");
@@ -227,7 +227,7 @@ void sm_token_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor
                                  (int)vc.size(2), (int)vhead, (int)Dv, block_tables.data_ptr<int>(), (int)block_tables.size(1),
                                  positions.data_ptr<int>(), token_seq.data_ptr<int>(), (int)n_rows, (int)H, (int)G, (float)scale,
                                  (int)window, opt_f32(temp, "temp", H), opt_f32(r1, "r1", H), opt_f32(r2, "r2", H), bf, nsplit,
-                                 nsplit > 1 ? part.data_ptr<float>() : nullptr, gp, g_ts, cur_stream(q1));
+                                 nsplit > 1 ? part.data_ptr<float>() : nullptr, gp, g_ts, opt_f32(sink, "sink", H), cur_stream(q1));
 }
 
 // Decode rows (the first `rows` tokens) of a mixer whose heads share key / value heads in groups of 8 or more, heads as the
@@ -236,7 +236,7 @@ bool sm_head_decode_attention(Tensor out, const Tensor& q1, const c10::optional<
                               const c10::optional<Tensor>& v_cache, const Tensor& block_tables, const Tensor& positions,
                               const Tensor& token_seq, int64_t G, int64_t Dv, double scale, int64_t window,
                               const c10::optional<Tensor>& temp, const c10::optional<Tensor>& r1, const c10::optional<Tensor>& r2,
-                              int64_t rows, const c10::optional<Tensor>& gate) {
+                              int64_t rows, const c10::optional<Tensor>& gate, const c10::optional<Tensor>& sink) {
   TORCH_CHECK(q1.is_cuda() && q1.scalar_type() == at::kBFloat16 && q1.dim() == 3 && q1.stride(2) == 1, "q1 must be bfloat16 [T, H, D1]");
   const int64_t T = q1.size(0), H = q1.size(1), D1 = q1.size(2);
   TORCH_CHECK(rows >= 0 && rows <= T, "rows past the batch");
@@ -277,7 +277,7 @@ bool sm_head_decode_attention(Tensor out, const Tensor& q1, const c10::optional<
                                               vc.data_ptr(), (int)vc.size(2), (int)vhead, (int)Dv, block_tables.data_ptr<int>(),
                                               (int)block_tables.size(1), positions.data_ptr<int>(), token_seq.data_ptr<int>(), (int)rows,
                                               (int)H, (int)G, (float)scale, (int)window, opt_f32(temp, "temp", H), opt_f32(r1, "r1", H),
-                                              opt_f32(r2, "r2", H), nsplit, nsplit > 1 ? part.data_ptr<float>() : nullptr, gp, g_ts,
+                                              opt_f32(r2, "r2", H), nsplit, nsplit > 1 ? part.data_ptr<float>() : nullptr, gp, g_ts, opt_f32(sink, "sink", H),
                                               cur_stream(q1));
 }
 
@@ -287,7 +287,7 @@ bool sm_tile_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor>
                        const c10::optional<Tensor>& v_cache, const Tensor& block_tables, const Tensor& seq_lens, const Tensor& qsl,
                        const Tensor& tile_seq, const Tensor& tile_q0, int64_t num_tiles, const c10::optional<Tensor>& counts, int64_t G,
                        int64_t Dv, double scale, int64_t window, const c10::optional<Tensor>& temp, const c10::optional<Tensor>& r1,
-                       const c10::optional<Tensor>& r2, const c10::optional<Tensor>& gate) {
+                       const c10::optional<Tensor>& r2, const c10::optional<Tensor>& gate, const c10::optional<Tensor>& sink) {
   TORCH_CHECK(q1.is_cuda() && q1.scalar_type() == at::kBFloat16 && q1.dim() == 3 && q1.stride(2) == 1, "q1 must be bfloat16 [T, H, D1]");
   const int64_t T = q1.size(0), H = q1.size(1), D1 = q1.size(2);
   int64_t D2 = 0;
@@ -333,7 +333,7 @@ bool sm_tile_attention(Tensor out, const Tensor& q1, const c10::optional<Tensor>
                                        (int)vc.size(2), (int)vhead, (int)Dv, block_tables.data_ptr<int>(), (int)block_tables.size(1),
                                        seq_lens.data_ptr<int>(), qsl.data_ptr<int>(), tile_seq.data_ptr<int>(), tile_q0.data_ptr<int>(),
                                        (int)num_tiles, cnt, (int)H, (int)G, (float)scale, (int)window, opt_f32(temp, "temp", H),
-                                       opt_f32(r1, "r1", H), opt_f32(r2, "r2", H), gp, g_ts, cur_stream(q1));
+                                       opt_f32(r1, "r1", H), opt_f32(r2, "r2", H), gp, g_ts, opt_f32(sink, "sink", H), cur_stream(q1));
 }
 
 Tensor sm_lightning_scan(const Tensor& qkvg, Tensor state, const Tensor& positions, const Tensor& qsl, const Tensor& state_slots,

@@ -582,6 +582,7 @@ void ar_all_gather(int64_t st, const Tensor& inp, Tensor out) {
 #include "seqmix_bindings.h"
 #include "dualmix_bindings.h"
 #include "hypermix_bindings.h"
+#include "recurmix_bindings.h"
 
 }  // namespace
 
@@ -600,15 +601,15 @@ TORCH_LIBRARY(dli, m) {
         "Tensor slot_mapping, Tensor(b!) cache, int H, int D, int R, int C) -> ()", &sm_latent_prep);
   m.def("sm_token_attention(Tensor(a!) out, Tensor q1, Tensor? q2, Tensor k_cache, Tensor? v_cache, Tensor block_tables, "
         "Tensor positions, Tensor token_seq, int G, int Dv, float scale, int window, Tensor? temp, Tensor? r1, Tensor? r2, int rows=-1, "
-        "Tensor? gate=None) -> ()",
+        "Tensor? gate=None, Tensor? sink=None) -> ()",
         &sm_token_attention);
   m.def("sm_head_decode_attention(Tensor(a!) out, Tensor q1, Tensor? q2, Tensor k_cache, Tensor? v_cache, Tensor block_tables, "
         "Tensor positions, Tensor token_seq, int G, int Dv, float scale, int window, Tensor? temp, Tensor? r1, Tensor? r2, int rows, "
-        "Tensor? gate=None) -> bool",
+        "Tensor? gate=None, Tensor? sink=None) -> bool",
         &sm_head_decode_attention);
   m.def("sm_tile_attention(Tensor(a!) out, Tensor q1, Tensor? q2, Tensor k_cache, Tensor? v_cache, Tensor block_tables, Tensor seq_lens, "
         "Tensor qsl, Tensor tile_seq, Tensor tile_q0, int num_tiles, Tensor? counts, int G, int Dv, float scale, int window, "
-        "Tensor? temp, Tensor? r1, Tensor? r2, Tensor? gate=None) -> bool", &sm_tile_attention);
+        "Tensor? temp, Tensor? r1, Tensor? r2, Tensor? gate=None, Tensor? sink=None) -> bool", &sm_tile_attention);
   m.def("sm_lightning_scan(Tensor qkvg, Tensor(a!) state, Tensor positions, Tensor qsl, Tensor state_slots, Tensor counts, "
         "int num_seqs, int H, int D, int Dv, Tensor decay, Tensor? tile_seq=None, Tensor? tile_q0=None, int num_tiles=0, "
         "bool plain_act=False) -> Tensor", &sm_lightning_scan);
@@ -630,13 +631,23 @@ TORCH_LIBRARY(dli, m) {
   m.def("dm_sigmoid_route(Tensor h, Tensor router, int E, int K, float scale) -> (Tensor, Tensor, Tensor)", &dm_sigmoid_route);
   m.def("dm_relu2_experts(Tensor h, Tensor ids, Tensor wts, Tensor up, Tensor down, bool gated=False) -> Tensor", &dm_relu2_experts);
   m.def("hm_stream_mix_norm(Tensor(a!) x, Tensor? y, Tensor? mix, Tensor? out_w, Tensor? in_w, Tensor? norm_w, float eps, float w_offset, "
-        "bool out_bf16) -> Tensor", &hm_stream_mix_norm);
+        "bool out_bf16, bool center=False) -> Tensor", &hm_stream_mix_norm);
   m.def("hm_causal_conv_add(Tensor h, Tensor w, Tensor(a!) state, Tensor positions, Tensor token_seq, Tensor qsl, Tensor state_slots, "
         "Tensor counts, int num_seqs, bool out_bf16) -> Tensor", &hm_causal_conv_add);
   m.def("hm_retention_prep(Tensor qkvg, Tensor positions, Tensor? freq, int rot_dims, int H, int D, int Dv, float k_scale) -> Tensor",
         &hm_retention_prep);
   m.def("hm_act_mul(Tensor x, bool silu) -> Tensor", &hm_act_mul);
-  m.def("hm_softmax_route(Tensor h, Tensor router, Tensor? bias, int K) -> (Tensor, Tensor)", &hm_softmax_route);
+  m.def("hm_softmax_route(Tensor h, Tensor router, Tensor? bias, int K, bool all=False) -> (Tensor, Tensor)", &hm_softmax_route);
+  m.def("rm_causal_conv(Tensor x, Tensor w, Tensor? bias, Tensor(a!) state, Tensor positions, Tensor token_seq, Tensor qsl, "
+        "Tensor state_slots, Tensor counts, int num_seqs, bool out_bf16) -> Tensor", &rm_causal_conv);
+  m.def("rm_rglru_scan(Tensor z, Tensor u, Tensor y, Tensor gate_bias, Tensor rate, Tensor(a!) state, Tensor positions, Tensor qsl, "
+        "Tensor state_slots, Tensor counts, int num_seqs, bool out_bf16) -> Tensor", &rm_rglru_scan);
+  m.def("rm_latent_norm_cache(Tensor proj, int Q, Tensor qw, Tensor? cw, float eps, Tensor positions, Tensor freq, float mag, "
+        "int rot_dims, Tensor slot_mapping, Tensor(a!)? cache, int C, int R) -> Tensor", &rm_latent_norm_cache);
+  m.def("rm_rotate_heads(Tensor(a!) q, Tensor positions, Tensor freq, float mag, int rot_dims, int H, int D, int R) -> ()",
+        &rm_rotate_heads);
+  m.def("rm_gate_heads(Tensor o, Tensor gate) -> Tensor", &rm_gate_heads);
+  m.def("rm_clamped_experts(Tensor h, Tensor ids, Tensor wts, Tensor gate_up, Tensor down, float limit) -> Tensor", &rm_clamped_experts);
   m.def("dm_relu2_rows(Tensor x) -> Tensor", &dm_relu2_rows);
   m.def("dm_set_grouped_experts(bool on) -> ()", &dm_set_grouped_experts);
   m.def("dm_gated_combine(Tensor(a!) x, float mult, Tensor p0, Tensor p1, float s0, float s1, Tensor g1, Tensor b1, Tensor? ff, "

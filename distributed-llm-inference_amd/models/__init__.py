@@ -20,10 +20,11 @@ from .llama import LlamaForCausalLM
 from .opt import OPTForCausalLM
 from .rodelix import RodelixForCausalLM
 from .sevelorn import SevelornForCausalLM
+from .sinilorn import SinilornForCausalLM
 from .vibunex import VibunexForCausalLM
 
 _ARCH = {"llama": LlamaForCausalLM, "mixtral": LlamaForCausalLM, "opt": OPTForCausalLM, "rodelix": RodelixForCausalLM,
-         "vibunex": VibunexForCausalLM, "sevelorn": SevelornForCausalLM}
+         "vibunex": VibunexForCausalLM, "sevelorn": SevelornForCausalLM, "sinilorn": SinilornForCausalLM}
 
 
 def torch_dtype(name: str) -> torch.dtype:

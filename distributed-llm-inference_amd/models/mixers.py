@@ -379,8 +379,128 @@ class Retention(nn.Module):
         return ops.linear(y, self.o.data)
 
 
+class GatedLinearRecurrence(nn.Module):
+    """``W_o (S ⊙ gelu_tanh(W_y h + b_y))`` with ``S`` the per-channel fp32 state of ``S ← a ⊙ S + sqrt(1 - a²) ⊙ i ⊙ u``:
+    ``u`` = causal convolution (``conv_taps`` taps, bias) of ``W_x h + b_x``; recurrence gate ``r`` and input gate ``i`` are
+    sigmoids of block-diagonal maps of ``u`` (``heads`` blocks of ``dim`` channels, biases); ``a = exp(-8 · r · softplus(λ))``."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, ctx: ParallelContext, dtype, device):
+        super().__init__()
+        self.s, self.dtype = spec, dtype
+        B, n, taps = spec.heads, spec.dim, spec.conv_taps
+        C = B * n
+        assert taps >= 1, "the convolution has at least the current token's tap"
+        self.yx, self.yx_b = _matrix(2 * C, width, ctx, dtype, device), Weight((2 * C,), None, ctx, dtype, device)
+        self.conv, self.conv_b = _param((C, taps), ctx, device), _param((C,), ctx, device)
+        self.gates = Weight((2 * B, n, n), None, ctx, dtype, device)        # the blocks of the recurrence gate, then those of the input gate
+        self.gates_b = _param((2, C), ctx, device)
+        self.lam = _param((C,), ctx, device)
+        self.o = _matrix(width, C, ctx, dtype, device)
+        self._taps = self._rate = self._gates_t = None                     # derived at first use (after loading)
+
+    def weights(self, p):
+        B = self.s.heads
+        yield p + "yx", self.yx, "normal", [p + "y", p + "x"]
+        yield p + "yx.b", self.yx_b, "zeros", [p + "y.b", p + "x.b"]
+        yield p + "conv", self.conv, "small", None
+        yield p + "conv.b", self.conv_b, "zeros", None
+        yield p + "gates", self.gates, "normal", [p + "ra", p + "ri"]
+        yield p + "gates.b", self.gates_b, "zeros", [p + "ra.b", p + "ri.b"]
+        yield p + "lam", self.lam, "small", None
+        yield p + "o", self.o, "normal", None
+
+    def cache(self, num_blocks, num_slots, dtype, device) -> LayerCache:
+        B, n, taps = self.s.heads, self.s.dim, self.s.conv_taps
+        return LayerCache(state=torch.zeros(num_slots, B * n, dtype=torch.float32, device=device),
+                          shift=torch.zeros(num_slots, max(taps - 1, 0), B * n, dtype=torch.float32, device=device))
+
+    def forward(self, h, meta, cache: LayerCache):
+        B, n = self.s.heads, self.s.dim
+        C = B * n
+        T = h.shape[0]
+        if self._taps is None:
+            self._taps = self.conv.data.t().contiguous()
+            self._rate = 8.0 * torch.nn.functional.softplus(self.lam.data)
+            # checkpoint order is [ra blocks | ri blocks]; the product wants a block's two gates side by side: [B, n, 2n]
+            g = self.gates.data.view(2, B, n, n)
+            self._gates_t = torch.cat([g[0].transpose(1, 2), g[1].transpose(1, 2)], dim=2).contiguous()
+        yx = ops.linear(h, self.yx.data, self.yx_b.data)
+        u = seqmix.causal_conv(yx[:, C:], self._taps, self.conv_b.data, cache.shift, meta, self.dtype)
+        z = torch.bmm(u.view(T, B, n).transpose(0, 1), self._gates_t)                      # [B, T, 2n]
+        out = seqmix.rglru_scan(z, u, yx[:, :C], self.gates_b.data, self._rate, cache.state, meta, self.dtype)
+        return ops.linear(out, self.o.data)
+
+
+class GatedLatentAttention(nn.Module):
+    """Latent attention behind a normed query latent: ``c_q = rms(W_dq h)``, ``q = W_uq c_q``; keys and values are expanded from
+    the cached latent ``c = rms(W_dkv h)[:C]`` and one rotated key part shared by the heads (the key expansion folded into
+    the query, the value expansion applied after the softmax, so the cache rows are all the attention kernel reads).
+    Half-split rotation with optionally stretched frequencies, sliding window, a per-head sink in the softmax denominator,
+    element-wise sigmoid output gate ``W_g h``.  ``spec.kv_from`` ≥ 0: no ``W_dkv``; the layer reads that layer's cache rows."""
+
+    def __init__(self, spec: MixerSpec, width: int, eps: float, ctx: ParallelContext, dtype, device):
+        super().__init__()
+        self.s, self.eps = spec, eps
+        H, D, R, Dv, C, Q = spec.heads, spec.dim, spec.rot_dim, spec.vdim, spec.kv_rank, spec.q_rank
+        assert spec.rot_dims <= R and spec.rot_dims % 2 == 0
+        self.own_kv = spec.kv_from < 0
+        kv = C + R if self.own_kv else 0
+        used = Q + kv + H * Dv
+        self.cols = (Q, kv, H * Dv, -used % 8)                  # query latent | latent + key part | output gate | alignment rows
+        self.down = _matrix(sum(self.cols), width, ctx, dtype, device)
+        self.q_norm = _param((Q,), ctx, device)
+        self.c_norm = _param((C,), ctx, device) if self.own_kv else None
+        self.uq = _matrix(H * (D + R), Q, ctx, dtype, device)
+        self.uk = _matrix(H * D, C, ctx, dtype, device)
+        self.uv = _matrix(H * Dv, C, ctx, dtype, device)
+        self.sink = _param((H,), ctx, device) if spec.sink else None
+        self.o = _matrix(width, H * Dv, ctx, dtype, device)
+        freq, self.mag = seqmix.stretched_inv_freq(spec.rot_base, spec.rot_dims, spec.rot_scaling, device)
+        self.register_buffer("inv_freq", freq, persistent=False)
+
+    def weights(self, p):
+        pad = [f"@zeros:{self.cols[3]}"] if self.cols[3] else []
+        yield p + "down", self.down, "normal", [p + "dq"] + ([p + "dkv"] if self.own_kv else []) + [p + "g"] + pad
+        yield p + "dq.norm", self.q_norm, "ones", None
+        if self.own_kv:
+            yield p + "dkv.norm", self.c_norm, "ones", None
+        yield p + "uq", self.uq, "normal", None
+        yield p + "uk", self.uk, "normal", None
+        yield p + "uv", self.uv, "normal", None
+        if self.sink is not None:
+            yield p + "sink", self.sink, "zeros", None
+        yield p + "o", self.o, "normal", None
+
+    def cache(self, num_blocks, num_slots, dtype, device) -> LayerCache:
+        s = self.s
+        if not self.own_kv:
+            return LayerCache(owns_pages=False)
+        return LayerCache(k=torch.zeros(num_blocks, KV_BLOCK_SIZE, s.kv_rank + s.rot_dim, dtype=dtype, device=device))
+
+    def forward(self, h, meta, cache: LayerCache):
+        s = self.s
+        H, D, R, Dv, C, Q = s.heads, s.dim, s.rot_dim, s.vdim, s.kv_rank, s.q_rank
+        T = h.shape[0]
+        nq, nkv, ng, _pad = self.cols
+        both = ops.linear(h, self.down.data)
+        cq = seqmix.latent_norm_cache(both, Q, self.q_norm.data, self.c_norm.data if self.own_kv else None, self.eps, meta.positions,
+                                      self.inv_freq, self.mag, s.rot_dims, meta.slot_mapping, cache.k if self.own_kv else None, C, R)
+        q = ops.linear(cq, self.uq.data)
+        seqmix.rotate_heads(q, meta.positions, self.inv_freq, self.mag, s.rot_dims, H, D, R)
+        q3 = q.view(T, H, D + R)
+        # key expansion folded into the query: (W_uk c) · q = c · (W_ukᵀ q) — one [D] → [C] product per head and token
+        q_lat = torch.bmm(q3[:, :, :D].transpose(0, 1), self.uk.data.view(H, D, C))                  # [H, T, C]
+        o_lat = torch.zeros(H, T, C, dtype=h.dtype, device=h.device)     # padding rows of a captured step stay zero
+        seqmix.token_attention(o_lat.transpose(0, 1), q_lat.transpose(0, 1), q3[:, :, D:], cache.k, None, meta, 1, C, s.scale,
+                               s.window, sink=self.sink.data if self.sink is not None else None)
+        # value expansion after the softmax: Σ p_j (W_uv c_j) = W_uv (Σ p_j c_j)
+        out = torch.bmm(o_lat, self.uv.data.view(H, Dv, C).transpose(1, 2))                          # [H, T, Dv]
+        return ops.linear(seqmix.gate_heads(out, both[:, nq + nkv:nq + nkv + ng]), self.o.data)
+
+
 MIXERS = {"gated_attention": GatedAttention, "retention": Retention, "attention": WindowAttention, "latent_attention": LatentAttention, "lightning": LightningAttention,
-          "sink_attention": SinkTalkAttention, "time_mix": TimeMix, "parallel": DualMixer}
+          "sink_attention": SinkTalkAttention, "time_mix": TimeMix, "parallel": DualMixer, "rglru": GatedLinearRecurrence,
+          "gated_latent_attention": GatedLatentAttention}
 
 
 class DenseFF(nn.Module):
@@ -436,17 +556,24 @@ class RoutedFF(nn.Module):
 class GatedDenseFF(nn.Module):
     """``W_down · (act(W_gate h) ⊙ W_up h)``; gate and up rows are one GEMM."""
 
-    def __init__(self, width: int, ff: int, act: str, ctx, dtype, device):
+    def __init__(self, width: int, ff: int, act: str, ctx, dtype, device, bias: bool = False):
         super().__init__()
         self.act = act
         self.gate_up, self.down = _matrix(2 * ff, width, ctx, dtype, device), _matrix(width, ff, ctx, dtype, device)
+        self.gate_up_b = Weight((2 * ff,), None, ctx, dtype, device) if bias else None
+        self.down_b = Weight((width,), None, ctx, dtype, device) if bias else None
 
     def weights(self, p):
         yield p + "gate_up", self.gate_up, "normal", [p + "gate", p + "up"]
         yield p + "down", self.down, "normal", None
+        if self.gate_up_b is not None:
+            yield p + "gate_up.b", self.gate_up_b, "zeros", [p + "gate.b", p + "up.b"]
+            yield p + "down.b", self.down_b, "zeros", None
 
     def forward(self, h):
-        return ops.linear(seqmix.act_mul(ops.linear(h, self.gate_up.data), self.act), self.down.data)
+        if self.gate_up_b is None:
+            return ops.linear(seqmix.act_mul(ops.linear(h, self.gate_up.data), self.act), self.down.data)
+        return ops.linear(seqmix.act_mul(ops.linear(h, self.gate_up.data, self.gate_up_b.data), self.act), self.down.data, self.down_b.data)
 
 
 class SoftmaxRoutedFF(nn.Module):
@@ -475,6 +602,32 @@ class SoftmaxRoutedFF(nn.Module):
         return seqmix.gated_experts(h, ids, wts, self.gate_up.data, self.down.data)
 
 
+class ScoreRoutedFF(nn.Module):
+    """``Σ_chosen w_e · expert_e(h)``: scores are the fp32 softmax of ``W_r h`` over all router outputs; the ``top`` outputs with
+    the largest ``score + correction`` are chosen and weigh ``score / Σ_chosen score``.  The last ``identity_experts`` outputs
+    are experts without tensors that return ``h`` itself; the others are clamped gated experts
+    ``W_down (g · sigmoid(1.702 g) · (u + 1))`` with ``g = min(W_gate h, limit)``, ``u = clamp(W_up h, ±limit)``."""
+
+    def __init__(self, spec: MixerSpec, width: int, ctx, dtype, device):
+        super().__init__()
+        self.s = spec
+        E, F, I = spec.experts, spec.ff, spec.identity_experts
+        assert 1 <= spec.top <= E + I and spec.ff_limit > 0.0
+        self.gate_up, self.down = Weight((E, 2 * F, width), None, ctx, dtype, device), Weight((E, width, F), None, ctx, dtype, device)
+        self.router, self.correction = _param((E + I, width), ctx, device), _param((E + I,), ctx, device)
+
+    def weights(self, p):
+        E = self.s.experts
+        yield p + "experts.gate_up", self.gate_up, "normal", [[p + f"e{e}.gate", p + f"e{e}.up"] for e in range(E)]
+        yield p + "experts.down", self.down, "normal", [[p + f"e{e}.down"] for e in range(E)]
+        yield p + "router", self.router, "normal", None
+        yield p + "correction", self.correction, "zeros", None
+
+    def forward(self, h):
+        ids, wts = seqmix.softmax_all_route(h, self.router.data, self.correction.data, self.s.top)
+        return seqmix.gated_experts(h, ids, wts, self.gate_up.data, self.down.data, limit=self.s.ff_limit)
+
+
 class StreamLinks(nn.Module):
     """How one sublayer reads and writes ``S`` copies of the stream: ``u = Σ_s in[s] x_s`` goes in; the result ``y`` comes back
     as ``x_t ← Σ_s mix[s, t] x_s + out[t] y``.  ``S = 1`` with all-ones weights is the plain residual sum."""
@@ -499,9 +652,14 @@ class HyperLayer(nn.Module):
     causal per-channel convolution over the sequence's last ``taps`` inputs (``taps`` = 0: none).  ``links`` False: one stream,
     plain residual sums (the link weights stay at one and are not part of a checkpoint)."""
 
-    def __init__(self, spec: MixerSpec, width: int, eps: float, streams: int, taps: int, ctx: ParallelContext, dtype, device):
+    def __init__(self, spec: MixerSpec, width: int, eps: float, streams: int, taps: int, ctx: ParallelContext, dtype, device,
+                 norm: str = "rms_offset"):
         super().__init__()
+        if norm not in ("rms_offset", "layer"):
+            raise ValueError(f"unknown norm {norm!r}")
         self.spec, self.eps, self.dtype, self.taps = spec, eps, dtype, taps
+        # "rms_offset": u / rms(u) · (1 + w); "layer": (u - mean) / sqrt(var + eps) · w
+        self.center, self.w_offset = norm == "layer", 0.0 if norm == "layer" else 1.0
         self.links = streams > 0
         S = max(streams, 1)
         self.norm1, self.hc1 = _param((width,), ctx, device), StreamLinks(S, ctx, device)
@@ -512,21 +670,24 @@ class HyperLayer(nn.Module):
         if spec.ff:
             self.norm2, self.hc2 = _param((width,), ctx, device), StreamLinks(S, ctx, device)
             if spec.ff_kind == "moe":
-                if spec.router != "softmax":
+                if spec.router == "softmax":
+                    self.ff = SoftmaxRoutedFF(spec, width, ctx, dtype, device)
+                elif spec.router == "softmax_all":
+                    self.ff = ScoreRoutedFF(spec, width, ctx, dtype, device)
+                else:
                     raise ValueError(f"hyper-connected layers route by softmax, not {spec.router!r}")
-                self.ff = SoftmaxRoutedFF(spec, width, ctx, dtype, device)
             else:
-                self.ff = GatedDenseFF(width, spec.ff, spec.ff_act, ctx, dtype, device)
+                self.ff = GatedDenseFF(width, spec.ff, spec.ff_act, ctx, dtype, device, bias=spec.ff_bias)
 
     def weights(self, p):
-        yield p + "norm1", self.norm1, "zeros", None
+        yield p + "norm1", self.norm1, "ones" if self.center else "zeros", None
         if self.links:
             yield from self.hc1.weights(p + "hc1.")
         if self.conv is not None:
             yield p + "canon1", self.conv, "small", None
         yield from self.mixer.weights(p + "mix.")
         if self.ff is not None:
-            yield p + "norm2", self.norm2, "zeros", None
+            yield p + "norm2", self.norm2, "ones" if self.center else "zeros", None
             if self.links:
                 yield from self.hc2.weights(p + "hc2.")
             yield from self.ff.weights(p + "mlp.")
@@ -534,6 +695,7 @@ class HyperLayer(nn.Module):
     def cache(self, num_blocks, num_slots, dtype, device) -> LayerCache:
         c = self.mixer.cache(num_blocks, num_slots, dtype, device)
         if self.taps:               # the sequence's last taps-1 mixer inputs, oldest first
+            assert c.shift is None, "the layer's input convolution and the mixer both want the shift rows"
             c.shift = torch.zeros(num_slots, self.taps - 1, self.norm1.data.shape[0], dtype=torch.float32, device=device)
         return c
 
@@ -541,7 +703,7 @@ class HyperLayer(nn.Module):
         """Write the previous sublayer's ``y`` back through its links ``prev`` (if any) and return this layer's mixer input
         before the convolution."""
         return seqmix.stream_mix_norm(x, y, prev.mix.data if prev else None, prev.w_out.data if prev else None, self.hc1.w_in.data,
-                                      self.norm1.data, self.eps, 1.0, out_dtype)
+                                      self.norm1.data, self.eps, self.w_offset, out_dtype, self.center)
 
     def forward(self, x, h, meta, cache: LayerCache):
         """``x``: fp32 streams ``[T, S, W]``, updated in place; ``h``: this layer's normed mixer input (``read``).  Returns the
@@ -553,8 +715,8 @@ class HyperLayer(nn.Module):
         y = self.mixer(h, meta, cache)
         if self.ff is None:
             return y, self.hc1
-        h2 = seqmix.stream_mix_norm(x, y, self.hc1.mix.data, self.hc1.w_out.data, self.hc2.w_in.data, self.norm2.data, self.eps, 1.0,
-                                    self.dtype)
+        h2 = seqmix.stream_mix_norm(x, y, self.hc1.mix.data, self.hc1.w_out.data, self.hc2.w_in.data, self.norm2.data, self.eps,
+                                    self.w_offset, self.dtype, self.center)
         return self.ff(h2), self.hc2
 
 

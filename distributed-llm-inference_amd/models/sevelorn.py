@@ -38,7 +38,7 @@ class SevelornForCausalLM(nn.Module):
         W = cfg.hidden_size
         self.streams = max(cfg.streams, 1)
         self.embed = Weight((cfg.vocab_size, W), None, ctx, dtype, device)
-        self.layers = nn.ModuleList(HyperLayer(s, W, cfg.rms_eps, cfg.streams, cfg.conv_taps, ctx, dtype, device)
+        self.layers = nn.ModuleList(HyperLayer(s, W, cfg.rms_eps, cfg.streams, cfg.conv_taps, ctx, dtype, device, cfg.stream_norm)
                                     for s in cfg.layer_specs)
         self.final_norm = _param((W,), ctx, device)
         self.head = Weight((cfg.vocab_size, W), None, ctx, dtype, device)
@@ -75,20 +75,22 @@ class SevelornForCausalLM(nn.Module):
             y, links = layer(x, h, meta, cache)
         # the last write-back, the sum of the streams and the closing norm in one pass
         h = seqmix.stream_mix_norm(x, y, links.mix.data if links else None, links.w_out.data if links else None, self.sum_w,
-                                   self.final_norm.data, self.cfg.rms_eps, 1.0, self.dtype)
+                                   self.final_norm.data, self.cfg.rms_eps, 0.0 if self.cfg.stream_norm == "layer" else 1.0, self.dtype,
+                                   self.cfg.stream_norm == "layer")
         if self.layer_outputs is not None:
             self.layer_outputs.append(x.sum(1))
         return h
 
     def compute_logits(self, h: torch.Tensor) -> torch.Tensor:
-        return ops.linear(h, self.head.data).float()
+        logits = ops.linear(h, self.head.data).float()
+        return logits.mul_(self.cfg.logit_scale) if self.cfg.logit_scale != 1.0 else logits
 
     # ---- parameters: (name, holder, init kind, checkpoint tensors: concatenated along dim 0, or — a list of lists — stacked)
     def named_weight_sources(self):
         yield "embed", self.embed, "normal", None
         for i, l in enumerate(self.layers):
             yield from l.weights(f"l{i}.")
-        yield "final.norm", self.final_norm, "zeros", None
+        yield "final.norm", self.final_norm, "ones" if self.cfg.stream_norm == "layer" else "zeros", None
         yield "head", self.head, "normal", None
 
     def named_weights(self):

@@ -192,7 +192,8 @@ def latent_prep(q: torch.Tensor, dkv: torch.Tensor, cw: torch.Tensor, eps: float
 def token_attention(out: torch.Tensor, q1: torch.Tensor, q2: Optional[torch.Tensor], k_cache: torch.Tensor,
                     v_cache: Optional[torch.Tensor], meta, G: int, Dv: int, scale: float, window: int = 0,
                     temp: Optional[torch.Tensor] = None, r1: Optional[torch.Tensor] = None,
-                    r2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    r2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                    sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Softmax attention of this step's tokens over their sequences' cached rows (which already hold this step's keys).
 
     ``q1 [T, H, D1]`` (and ``q2 [T, H, D2]``) against key rows ``[G, D1 + D2]``: ``score = (q1·k[:D1] + q2·k[D1:]) · scale ·
@@ -200,7 +201,8 @@ def token_attention(out: torch.Tensor, q1: torch.Tensor, q2: Optional[torch.Tens
     the values are the first ``Dv`` entries of the key rows (latent attention: the cached latent is key and value).
     ``window`` > 0: a query at position ``p`` sees positions ``p-window+1 … p``; 0: all up to ``p``.  ``gate [T, H]``
     (pre-activation, row-strided view): head ``h``'s result is multiplied by ``sigmoid(gate[t, h])``.  Views may be strided
-    (last dim contiguous).  Writes ``out [T, H, Dv]``."""
+    (last dim contiguous).  ``sink`` fp32 ``[H]``: the softmax denominator of head ``h`` also holds ``exp(sink[h])`` (a logit
+    without key or value, not scaled).  Writes ``out [T, H, Dv]``."""
     if _act_ok(q1):
         lib = _hip()
         rows = -1
@@ -208,17 +210,17 @@ def token_attention(out: torch.Tensor, q1: torch.Tensor, q2: Optional[torch.Tens
             # prefill chunks: 64-query tiles on the matrix cores; the per-token kernel keeps the decode rows in front
             if lib.sm_tile_attention(out, q1, q2, k_cache, v_cache, meta.block_tables, meta.seq_lens, meta.query_start_loc,
                                      meta.prefill_tile_seq, meta.prefill_tile_q0, meta.num_prefill_tiles,
-                                     meta.counts if meta.counts_on_device else None, G, Dv, scale, window, temp, r1, r2, gate):
+                                     meta.counts if meta.counts_on_device else None, G, Dv, scale, window, temp, r1, r2, gate, sink):
                 rows = meta.num_decode
         T, H = q1.shape[0], q1.shape[1]
         todo = T if rows < 0 else rows                       # tokens the tile kernel left (all of them in a pure decode step)
         if (HEAD_DECODE and todo > 0 and q1.dtype == torch.bfloat16 and H // G >= 8 and meta.num_prefill_tiles == (0 if rows < 0 else meta.num_prefill_tiles)
                 and lib.sm_head_decode_attention(out, q1, q2, k_cache, v_cache, meta.block_tables, meta.positions, meta.token_seq,
-                                                 G, Dv, scale, window, temp, r1, r2, todo, gate)):
+                                                 G, Dv, scale, window, temp, r1, r2, todo, gate, sink)):
             rows = 0                                         # done with the heads as matrix-core columns
         if rows != 0:
             lib.sm_token_attention(out, q1, q2, k_cache, v_cache, meta.block_tables, meta.positions, meta.token_seq,
-                                   G, Dv, scale, window, temp, r1, r2, rows, gate)
+                                   G, Dv, scale, window, temp, r1, r2, rows, gate, sink)
         return out
     T, H, D1 = q1.shape
     rowk = k_cache.shape[-1]
@@ -253,7 +255,11 @@ def token_attention(out: torch.Tensor, q1: torch.Tensor, q2: Optional[torch.Tens
         if window > 0:
             hidden = hidden | (dist >= window)
         s = s.masked_fill(hidden.unsqueeze(1), float("-inf"))
-        o = torch.einsum("nhl,lhd->nhd", torch.softmax(s, dim=-1), Vh)
+        if sink is not None:
+            pw = torch.softmax(torch.cat([s, sink.view(1, H, 1).expand(t1 - t0, H, 1)], dim=-1), dim=-1)[..., :-1]
+        else:
+            pw = torch.softmax(s, dim=-1)
+        o = torch.einsum("nhl,lhd->nhd", pw, Vh)
         if gate is not None:
             o = o * torch.sigmoid(gate[t0:t1].float()).unsqueeze(2)
         out[t0:t1] = o.to(out.dtype)
@@ -536,13 +542,14 @@ def gated_combine(x: torch.Tensor, mult: float, parts: list, scales: list, gate1
 # ``csrc/kernels/hypermix.hip`` (``torch.ops.dli.hm_*``) beside extensions of the kernels above.
 def stream_mix_norm(x: torch.Tensor, y: Optional[torch.Tensor], mix: Optional[torch.Tensor], out_w: Optional[torch.Tensor],
                     in_w: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], eps: float, w_offset: float,
-                    out_dtype: torch.dtype) -> Optional[torch.Tensor]:
+                    out_dtype: torch.dtype, center: bool = False) -> Optional[torch.Tensor]:
     """One pass over the fp32 streams ``x [T, S, W]``.  With ``y [T, W]`` (a sublayer's output): all streams at once from the
     old ones, in place, ``x[:, t] ← Σ_s mix[s, t] · x[:, s] + out_w[t] · y``.  With ``in_w [S]``: returns
     ``rms_norm(Σ_s in_w[s] · x[:, s]) · (w_offset + norm_w)`` in ``out_dtype`` — what the next sublayer (or the LM head)
-    reads, computed from the updated streams."""
+    reads, computed from the updated streams.  ``center``: a layer norm without bias instead — the mean is taken off first and
+    the statistic is the variance."""
     if x.is_cuda:
-        h = _hip().hm_stream_mix_norm(x, y, mix, out_w, in_w, norm_w, eps, w_offset, out_dtype == torch.bfloat16)
+        h = _hip().hm_stream_mix_norm(x, y, mix, out_w, in_w, norm_w, eps, w_offset, out_dtype == torch.bfloat16, center)
         return h if in_w is not None else None
     if y is not None:
         new = torch.einsum("st,nsw->ntw", mix, x) + out_w.view(1, -1, 1) * y.float().unsqueeze(1)
@@ -550,6 +557,8 @@ def stream_mix_norm(x: torch.Tensor, y: Optional[torch.Tensor], mix: Optional[to
     if in_w is None:
         return None
     u = torch.einsum("s,nsw->nw", in_w, x)
+    if center:
+        u = u - u.mean(-1, keepdim=True)
     return (u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps) * (w_offset + norm_w)).to(out_dtype)
 
 
@@ -624,10 +633,15 @@ def softmax_route(h: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Te
     return ids[:, :top].int(), torch.softmax(val[:, :top], dim=-1)
 
 
-def gated_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
+def gated_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
+                  limit: float = 0.0) -> torch.Tensor:
     """``Σ_slots wts[t, s] · down[e] · (silu(gate[e] · h[t]) ⊙ up[e] · h[t])`` with ``e = ids[t, s]``; ``gate_up [E, 2F, W]``
-    (an expert's gate rows, then its up rows), ``down [E, W, F]``."""
+    (an expert's gate rows, then its up rows), ``down [E, W, F]``.  ``limit`` > 0: the clamped form instead —
+    ``g = min(gate · h, limit)``, ``u = clamp(up · h, ±limit)``, activation ``g · sigmoid(1.702 g) · (u + 1)`` — and an id
+    ``e ≥ E`` names an identity expert, whose output is ``h[t]`` itself."""
     if _act_ok(h):
+        if limit > 0.0:
+            return _hip().rm_clamped_experts(h, ids, wts, gate_up, down, limit)
         return _hip().dm_relu2_experts(h, ids, wts, gate_up, down, True)
     F = gate_up.shape[1] // 2
     out = torch.zeros(h.shape[0], h.shape[1])
@@ -636,6 +650,139 @@ def gated_experts(h: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor, gate_up
         tok, slot = torch.nonzero(ids == e, as_tuple=True)
         if tok.numel():
             gu = hf[tok] @ gate_up[e].float().t()
-            a = (torch.nn.functional.silu(gu[:, :F]) * gu[:, F:]).to(h.dtype).float()
+            if limit > 0.0:
+                g, u = gu[:, :F].clamp(max=limit), gu[:, F:].clamp(-limit, limit)
+                a = (g * torch.sigmoid(1.702 * g) * (u + 1.0)).to(h.dtype).float()
+            else:
+                a = (torch.nn.functional.silu(gu[:, :F]) * gu[:, F:]).to(h.dtype).float()
             out.index_add_(0, tok, (a @ down[e].float().t()) * wts[tok, slot].unsqueeze(1))
+    if limit > 0.0:
+        out += hf * (wts * (ids >= gate_up.shape[0])).sum(-1, keepdim=True)
     return out.to(h.dtype)
+
+
+# ====================================================================================== gated recurrences, gated latent attention
+# Ops of stacks that alternate a gated linear recurrence per channel with latent attention behind a normed query latent
+# (``models/mixers.py``: ``GatedLinearRecurrence``, ``GatedLatentAttention``, ``ScoreRoutedFF``).  GPU kernels:
+# ``csrc/kernels/recurmix.hip`` (``torch.ops.dli.rm_*``) beside extensions of the kernels above.
+def causal_conv(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor, meta,
+                out_dtype: torch.dtype) -> torch.Tensor:
+    """``x [T, C]`` (a row-strided view); ``w [taps, C]`` fp32 (tap-major: the last row weighs the token itself).  Row ``t`` of
+    the result is ``bias + Σ_j w[j] · x[t - taps + 1 + j]`` over the rows of the same sequence: rows above inside a chunk, the
+    sequence's ``state`` rows ``[slots, taps-1, C]`` (its last ``taps-1`` inputs, oldest first) before a chunk's start, zero
+    before position 0.  The state rows are then moved on to the sequence's last ``taps-1`` inputs of this step."""
+    if _act_ok(x):
+        return _hip().rm_causal_conv(x, w, bias, state, meta.positions, meta.token_seq, meta.query_start_loc, meta.state_slots,
+                                     meta.counts, meta.num_seqs, out_dtype == torch.bfloat16)
+    taps, C = w.shape
+    xf = x.float()
+    out = torch.zeros(x.shape[0], C)
+    for _i, t0, t1, slot in _seq_rows(meta):
+        p0, n = int(meta.positions[t0]), t1 - t0
+        hist = state[slot].clone() if taps > 1 else xf.new_zeros(0, C)
+        for r in range(taps - 1):
+            if p0 - (taps - 1) + r < 0:
+                hist[r] = 0.0
+        ext = torch.cat([hist, xf[t0:t1]], dim=0)
+        for j in range(taps):
+            out[t0:t1] += w[j] * ext[j:j + n]
+        if taps > 1:
+            state[slot] = ext[n:]
+    if bias is not None:
+        out = out + bias
+    return out.to(out_dtype)
+
+
+def rglru_scan(z: torch.Tensor, u: torch.Tensor, y: torch.Tensor, gate_bias: torch.Tensor, rate: torch.Tensor, state: torch.Tensor,
+               meta, out_dtype: torch.dtype) -> torch.Tensor:
+    """The gated linear recurrence per channel.  ``z [B, T, 2·n]``: pre-activations of the recurrence gate (first ``n`` of a
+    block's row) and the input gate (last ``n``) of the ``B`` blocks of ``n`` channels, before their biases ``gate_bias`` fp32
+    ``[2, B·n]``; ``u [T, B·n]`` the recurrence's input; ``y [T, B·n]`` (row-strided view) the other branch before its
+    tanh-GELU; ``rate`` fp32 ``[B·n]`` = ``8 · softplus(λ)``.  Per sequence and channel, in fp32, token by token:
+    ``a = exp(-rate · sigmoid(z_r + b_r))``, ``S ← a · S + sqrt(1 - a²) · sigmoid(z_i + b_i) · u`` with ``S`` the sequence's
+    ``state[slot]`` row (zero at position 0), written back after the step's last token.  Returns ``S · gelu_tanh(y)``."""
+    if _act_ok(u):
+        return _hip().rm_rglru_scan(z, u, y, gate_bias, rate, state, meta.positions, meta.query_start_loc, meta.state_slots,
+                                    meta.counts, meta.num_seqs, out_dtype == torch.bfloat16)
+    B, T, n2 = z.shape
+    n = n2 // 2
+    zf = z.float().view(B, T, 2, n).permute(2, 1, 0, 3).reshape(2, T, B * n)
+    r, i = torch.sigmoid(zf[0] + gate_bias[0]), torch.sigmoid(zf[1] + gate_bias[1])
+    a = torch.exp(-rate * r)
+    b = torch.sqrt(1.0 - a * a) * i * u.float()
+    out = torch.zeros(T, B * n)
+    for _i, t0, t1, slot in _seq_rows(meta):
+        S = state[slot].clone() if int(meta.positions[t0]) > 0 else torch.zeros(B * n)
+        for t in range(t0, t1):
+            S = a[t] * S + b[t]
+            out[t] = S
+        state[slot] = S
+    return (out * torch.nn.functional.gelu(y.float(), approximate="tanh")).to(out_dtype)
+
+
+def _turn_half(v: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, mag: float, dims: int) -> torch.Tensor:
+    """fp32 ``[T, …, R]``: entries ``i`` and ``i + dims/2`` turned by ``position · inv_freq[i]``, cosine and sine times ``mag``."""
+    ang = positions.double()[:, None] * inv_freq[None, :]
+    cos, sin = (ang.cos() * mag).float(), (ang.sin() * mag).float()
+    while cos.dim() < v.dim():
+        cos, sin = cos.unsqueeze(1), sin.unsqueeze(1)
+    half = dims // 2
+    a, b = v[..., :half], v[..., half:dims]
+    return torch.cat([a * cos - b * sin, b * cos + a * sin, v[..., dims:]], dim=-1)
+
+
+def latent_norm_cache(proj: torch.Tensor, Q: int, qw: torch.Tensor, cw: Optional[torch.Tensor], eps: float, positions: torch.Tensor,
+                      inv_freq: torch.Tensor, mag: float, rot_dims: int, slot_mapping: torch.Tensor, cache: Optional[torch.Tensor],
+                      C: int, R: int) -> torch.Tensor:
+    """Leading columns of ``proj`` rows = ``[query latent (Q) | key / value latent (C) | shared key part (R)]``.  Returns the
+    query latent divided by its root mean square times ``qw`` (contiguous ``[T, Q]``).  With ``cache`` (token-major rows
+    ``[latent | rotated key]``): the key / value latent, divided by its root mean square times ``cw``, and the shared key
+    part, entries ``i`` and ``i + rot_dims/2`` turned by ``position · inv_freq[i]`` with cosine and sine times ``mag``, go to
+    the rows ``slot_mapping`` (< 0: skipped).  Without: the rows hold the query latent only."""
+    if _act_ok(proj):
+        return _hip().rm_latent_norm_cache(proj, Q, qw, cw, eps, positions, inv_freq, mag, rot_dims, slot_mapping, cache, C, R)
+    T = proj.shape[0]
+    cq = proj[:, :Q].float()
+    cq = (cq * torch.rsqrt((cq * cq).mean(-1, keepdim=True) + eps) * qw).to(proj.dtype)
+    if cache is not None:
+        c = proj[:, Q:Q + C].float()
+        c = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * cw
+        kr = _turn_half(proj[:, Q + C:Q + C + R].float(), positions[:T], inv_freq, mag, rot_dims)
+        keep = slot_mapping[:T] >= 0
+        cache.view(-1, C + R)[slot_mapping[:T][keep].long()] = torch.cat([c, kr], dim=-1)[keep].to(cache.dtype)
+    return cq
+
+
+def rotate_heads(q: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, mag: float, rot_dims: int, H: int, D: int,
+                 R: int) -> None:
+    """In place on ``q [T, H·(D+R)]``: in the last ``R`` entries of every head, entries ``i`` and ``i + rot_dims/2`` are
+    turned by ``position · inv_freq[i]`` with cosine and sine times ``mag`` (fp32 arithmetic)."""
+    if _act_ok(q):
+        _hip().rm_rotate_heads(q, positions, inv_freq, mag, rot_dims, H, D, R)
+        return
+    T = q.shape[0]
+    qv = q.view(T, H, D + R)
+    qv[:, :, D:] = _turn_half(qv[:, :, D:].float(), positions[:T], inv_freq, mag, rot_dims).to(q.dtype)
+
+
+def gate_heads(o: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """``o [H, T, Dv]`` (head-major) times ``sigmoid(gate [T, H·Dv])`` (pre-activation, row-strided view), as token-major
+    contiguous rows ``[T, H·Dv]``."""
+    if _act_ok(o):
+        return _hip().rm_gate_heads(o, gate)
+    H, T, Dv = o.shape
+    return (o.float().transpose(0, 1).reshape(T, H * Dv) * torch.sigmoid(gate.float())).to(o.dtype)
+
+
+def softmax_all_route(h: torch.Tensor, router: torch.Tensor, choice_bias: Optional[torch.Tensor], top: int):
+    """fp32 scores ``s = softmax(router · h)`` over ALL router outputs (``router`` fp32 ``[E, W]``); the ``top`` outputs with
+    the largest ``s + choice_bias`` are chosen (ties: lowest index) and weigh ``s / (Σ_chosen s + 1e-20)`` — the bias moves the
+    choice, not the weights.  Returns ``(ids int32 [T, top], weights fp32 [T, top])``."""
+    if _act_ok(h):
+        return _hip().hm_softmax_route(h, router, choice_bias, top, True)
+    sc = torch.softmax(h.float() @ router.t(), dim=-1)
+    ch = sc if choice_bias is None else sc + choice_bias
+    _val, ids = torch.sort(ch, dim=-1, descending=True, stable=True)
+    ids = ids[:, :top]
+    w = torch.gather(sc, 1, ids)
+    return ids.int(), w / (w.sum(-1, keepdim=True) + 1e-20)
