@@ -23,6 +23,15 @@ stacks (four fp32 streams, a four-tap input convolution) with their closest fami
 Mixtral expert width — beside ``mixtral``; ``sevelorn-retention`` = retention (heads of 128 × 128) + a tanh-GELU gated
 feed-forward of the Llama width — beside ``rodelix-lightning`` (mixer) and ``llama`` (feed-forward); ``sevelorn`` = an
 attention layer, an attention layer on the first one's keys / values (both with experts) and a retention layer (dense).
+
+``--models rodelix-lightning,sinilorn-recurrence,rodelix-latent_attention,sinilorn-latent,mixtral,sinilorn`` compares the
+Sinilorn stacks (four fp32 streams read through a layer norm) with their closest families: ``sinilorn-recurrence`` = a gated
+linear recurrence over ``width`` channels in blocks of 128 behind a four-tap convolution + a silu-gated dense feed-forward with
+biases of the Llama width — beside ``rodelix-lightning`` (the framework's other recurrent mixer); ``sinilorn-latent`` = gated
+latent attention (512-wide latent + 64 rotated, queries through a latent of 3/4 of the width, window 1024, sink, output gate)
++ 8 clamped experts and 2 identity experts, 2 per token, of the Mixtral expert width — beside ``rodelix-latent_attention``
+(mixer) and ``mixtral`` (experts); ``sinilorn`` = a recurrence (dense), a latent layer and a latent layer on the second
+one's cache rows (both with experts).
 """
 from __future__ import annotations
 
@@ -84,8 +93,23 @@ def sevelorn_raw(width, heads, kv, ffn, kinds):
             "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5}, "layers": [mk[k] for k in kinds]}
 
 
+def sinilorn_raw(width, heads, kv, ffn, kinds):
+    moe = {"kind": "moe", "expert": {"ff": ffn // 2, "limit": 7.0}, "router": {"experts": 8, "identity": 2, "top": 2}}
+    dense = {"kind": "dense", "ff": ffn}
+    lat = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": width * 3 // 4, "scale": 192 ** -0.5,
+           "mask": {"size": 1024},
+           "rot": {"base": 1000000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}
+    mk = {
+        "recurrence": {"type": "rglru", "mlp": dense, "mixer": {"blocks": width // 128, "conv": 4, "width": width}},
+        "latent": {"type": "latent_attention", "mlp": moe, "mixer": lat},
+        "shared_latent": {"type": "latent_attention", "mlp": moe, "mixer": dict(lat, kv_from=1)},
+    }
+    return {"architecture": "Sinilorn", "vocab": 32000, "width": width, "streams": 4, "logit_scale": 1.0, "norm": {"eps": 1e-5},
+            "layers": [mk[k] for k in kinds]}
+
+
 def model_configs(size):
-    from dli_amd.config import ModelConfig, rodelix_config, sevelorn_config, vibunex_config
+    from dli_amd.config import ModelConfig, rodelix_config, sevelorn_config, sinilorn_config, vibunex_config
     s = SIZES[size]
     out = {"llama": ModelConfig(name=f"llama-{size}", arch="llama", vocab_size=32000, hidden_size=s["width"],
                                 intermediate_size=s["ffn"], num_layers=LAYERS, num_heads=s["heads"], num_kv_heads=s["kv"],
@@ -97,6 +121,9 @@ def model_configs(size):
     for name, kinds in (("sevelorn", ("attention", "shared_attention", "retention")), ("sevelorn-attention", ("attention",) * LAYERS),
                         ("sevelorn-retention", ("retention",) * LAYERS)):
         out[name] = sevelorn_config(sevelorn_raw(s["width"], s["heads"], s["kv"], s["ffn"], kinds), name=f"{name}-{size}")
+    for name, kinds in (("sinilorn", ("recurrence", "latent", "shared_latent")), ("sinilorn-recurrence", ("recurrence",) * LAYERS),
+                        ("sinilorn-latent", ("latent",) * LAYERS)):
+        out[name] = sinilorn_config(sinilorn_raw(s["width"], s["heads"], s["kv"], s["ffn"], kinds), name=f"{name}-{size}")
     kinds = ("attention", "lightning", "latent_attention")
     out["rodelix"] = rodelix_config(rodelix_raw(s["width"], s["heads"], s["kv"], s["ffn"], kinds), name=f"rodelix-{size}")
     for k in kinds:

@@ -161,6 +161,8 @@ class ModelConfig:
         h, i, v, l = self.hidden_size, self.intermediate_size, self.vocab_size, self.num_layers
         if self.arch == "sevelorn":
             return 2 * v * h + h + sum(_hyper_layer_params(m, h, self.streams, self.conv_taps) for m in self.layer_specs)
+        if self.arch == "sinilorn":
+            return 2 * v * h + h + sum(_sinilorn_layer_params(m, h, self.streams) for m in self.layer_specs)
         if self.layer_specs:
             tot = 2 * v * h + 2 * h
             for m in self.layer_specs:
@@ -211,6 +213,23 @@ def _hyper_layer_params(m: MixerSpec, h: int, streams: int, taps: int) -> int:
         tot += h * m.heads * (2 * m.dim + 2 * m.vdim) + m.heads * m.vdim * h
     if m.ff:
         tot += h + hc + (m.experts * 3 * h * m.ff + m.experts * (h + 1) if m.ff_kind == "moe" else 3 * h * m.ff)
+    return tot
+
+
+def _sinilorn_layer_params(m: MixerSpec, h: int, streams: int) -> int:
+    """Parameters of one Sinilorn layer (norms, stream weights, mixer, feed-forward)."""
+    hc = (2 * streams + streams * streams) if streams else 0
+    tot = h + hc
+    if m.kind == "rglru":
+        c = m.heads * m.dim
+        tot += 2 * (c * h + c) + c * (m.conv_taps + 1) + 2 * (m.heads * m.dim * m.dim + c) + c + c * h
+    else:
+        kv = 0 if m.kv_from >= 0 else h * (m.kv_rank + m.rot_dim) + m.kv_rank
+        tot += h * m.q_rank + m.q_rank + m.q_rank * m.heads * (m.dim + m.rot_dim) + kv + m.kv_rank * m.heads * (m.dim + m.vdim) \
+            + m.heads + 2 * m.heads * m.vdim * h
+    if m.ff:
+        n_out = m.experts + m.identity_experts
+        tot += h + hc + (m.experts * 3 * h * m.ff + n_out * (h + 1) if m.ff_kind == "moe" else 3 * h * m.ff + 2 * m.ff + h)
     return tot
 
 
@@ -528,6 +547,19 @@ MODEL_PRESETS: dict[str, ModelConfig] = {
             {"type": "attention", "mlp": None,
              "mixer": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 24, "scale": 0.2, "kv_from": 1}}]},
         name="tiny-sevelorn", dtype="float32"),
+    # hyper-connected streams read through a layer norm; a gated linear recurrence, gated latent attention (one layer on
+    # another's cache rows), a biased dense and a score-routed feed-forward with identity experts
+    "tiny-sinilorn": sinilorn_config({
+        "vocab": 288, "width": 72, "streams": 2, "logit_scale": 0.75, "norm": {"eps": 1e-5},
+        "layers": [
+            {"type": "latent_attention", "mlp": {"kind": "moe", "expert": {"ff": 40, "limit": 2.0}, "router": {"experts": 3, "identity": 2, "top": 2}},
+             "mixer": {"heads": 3, "dim": 16, "rot_dim": 8, "vdim": 24, "kv_rank": 32, "q_rank": 40, "scale": 0.2, "mask": {"size": 37},
+                       "rot": {"base": 5000.0, "dims": 8, "scaling": {"factor": 2.0, "original": 64, "fast": 16.0, "slow": 2.0}}}},
+            {"type": "rglru", "mlp": {"kind": "dense", "ff": 96}, "mixer": {"blocks": 3, "conv": 4, "width": 48}},
+            {"type": "latent_attention", "mlp": None,
+             "mixer": {"heads": 2, "dim": 24, "rot_dim": 8, "vdim": 16, "kv_rank": 32, "q_rank": 24, "scale": 0.25, "kv_from": 0,
+                       "rot": {"base": 5000.0, "dims": 8, "scaling": {"factor": 2.0, "original": 64, "fast": 16.0, "slow": 2.0}}}}]},
+        name="tiny-sinilorn", dtype="float32"),
     "tiny-opt": ModelConfig(name="tiny-opt", arch="opt", vocab_size=512, hidden_size=64,
                             intermediate_size=128, num_layers=2, num_heads=4, num_kv_heads=4,
                             head_dim=16, max_position=512, pos_offset=2, tie_embeddings=True,

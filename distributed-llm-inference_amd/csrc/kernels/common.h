@@ -44,6 +44,17 @@ __device__ __forceinline__ uint16_t f2bf(float f) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
+// activation of a gated feed-forward: silu(gate) · up, or with limit > 0 the clamped form
+// g = min(gate, limit), u = clamp(up, ±limit): g · sigmoid(1.702 g) · (u + 1)
+__device__ __forceinline__ float gated_act(float gate, float up, float limit) {
+  if (limit > 0.f) {
+    gate = fminf(gate, limit);
+    up = fminf(fmaxf(up, -limit), limit);
+    return gate * fast_rcp(1.f + fast_exp2(-1.702f * 1.4426950408889634f * gate)) * (up + 1.f);
+  }
+  return gate * fast_rcp(1.f + fast_exp2(-1.4426950408889634f * gate)) * up;
+}
+
 // OCP e4m3 (gfx950 native) <-> float
 __device__ __forceinline__ float fp8_to_f(uint8_t v) {
   return __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(v), 0);

@@ -74,7 +74,7 @@ __global__ __launch_bounds__(512) void gemm256_kernel(
     const uint16_t* __restrict__ A, int64_t a_stride, const uint16_t* __restrict__ W, int64_t w_expert_stride,
     const int* __restrict__ sorted_ids, const int* __restrict__ tile_expert, const int* __restrict__ meta,
     const float* __restrict__ topk_w, int top_k, void* __restrict__ out_, int64_t out_stride, int M, int K, int N_half,
-    int n_col_blocks, int k_splits, int64_t slab_elems, int lin_begin, int lin_count) {
+    int n_col_blocks, int k_splits, int64_t slab_elems, int lin_begin, int lin_count, float act_limit) {
   uint16_t* out = reinterpret_cast<uint16_t*>(out_);
   __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE_BYTES];
 
@@ -339,7 +339,7 @@ __global__ __launch_bounds__(512) void gemm256_kernel(
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const float gate = acc[m][n][r], up = acc[m][n + 2][r];
-            o[r] = (short)f2bf(gate * fast_rcp(1.f + fast_exp2(-1.4426950408889634f * gate)) * up);
+            o[r] = (short)f2bf(gated_act(gate, up, act_limit));
           }
           *reinterpret_cast<bf16x4*>(dst + n * 16) = o;        // grouped padding rows hold finite junk, never read back
         }
@@ -377,7 +377,7 @@ __global__ __launch_bounds__(512) void gemm256_kernel(
 void launch_grouped_gemm256(int epilogue, const void* A, int64_t a_stride, const void* W, int64_t w_expert_stride,
                             const int* sorted_ids, const int* tile_expert, const int* meta, const float* topk_w, int top_k,
                             void* out, int64_t out_stride, int K, int N_out, int max_tiles, int k_splits, int64_t slab_elems,
-                            hipStream_t stream) {
+                            hipStream_t stream, float act_limit) {
   using namespace g256;
   if (max_tiles == 0) return;
   static const int half_tiles = [] {                                          // DLI_G256_HALF_TILES=0: every tile as a full tile (A/B)
@@ -390,7 +390,7 @@ void launch_grouped_gemm256(int epilogue, const void* A, int64_t a_stride, const
 #define G256_GO(EPI)                                                                                                       \
   hipLaunchKernelGGL((gemm256_kernel<EPI, true>), grid, dim3(512), 0, stream, (const uint16_t*)A, a_stride, (const uint16_t*)W, \
                      w_expert_stride, sorted_ids, tile_expert, meta, topk_w, top_k, out, out_stride, 0, K, N_out, n_col_blocks, \
-                     k_splits, slab_elems, half_tiles, 0)
+                     k_splits, slab_elems, half_tiles, 0, act_limit)
   if (epilogue == EPI_SWIGLU) G256_GO(EPI_SWIGLU);
   else if (epilogue == EPI_SCATTER) G256_GO(EPI_SCATTER);
   else G256_GO(EPI_SCATTER_SPLITK);
@@ -491,7 +491,7 @@ void launch_dense_gemm256(bool swiglu, const void* x, int64_t x_stride, const vo
 #define G256_DENSE(EPI, grid_, out_ptr_, ld_, splits_, slab_, begin_, count_)                                                    \
   hipLaunchKernelGGL((gemm256_kernel<EPI, false>), dim3(grid_), dim3(512), 0, stream, (const uint16_t*)x, x_stride,              \
                      (const uint16_t*)W, (int64_t)0, nullptr, nullptr, nullptr, nullptr, 1, out_ptr_, ld_, M, K, N_out,          \
-                     n_col_blocks, splits_, slab_, begin_, count_)
+                     n_col_blocks, splits_, slab_, begin_, count_, 0.f)
   if (k_splits > 1) {
     const int64_t ldc = (int64_t)N_out * (swiglu ? 2 : 1), slab = (int64_t)M * ldc;
     const int grid = (n_tiles * n_col_blocks * k_splits + 7) / 8 * 8;

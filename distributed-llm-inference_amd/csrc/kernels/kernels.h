@@ -10,7 +10,8 @@ void launch_rms_norm(void* out, const void* x, const void* w, float eps, int row
                      int64_t out_stride, hipStream_t stream);
 void launch_fused_add_rms_norm(void* x, void* residual, const void* w, float eps, int rows, int H, int64_t x_stride,
                                hipStream_t stream);
-void launch_silu_and_mul(void* out, const void* x, int rows, int inter, int64_t x_stride, hipStream_t stream);
+// act_limit > 0: the clamped gated activation min(g, limit) · sigmoid(1.702 ·) · (clamp(u, ±limit) + 1) instead of silu(g) · u
+void launch_silu_and_mul(void* out, const void* x, int rows, int inter, int64_t x_stride, hipStream_t stream, float act_limit = 0.f);
 void launch_rms_norm_quant(const void* x, void* residual, const void* w, float eps, int rows, int H, int64_t x_stride, void* q,
                            float* scales, hipStream_t stream);
 void launch_quant_rows_fp8(bool silu, const void* x, int64_t x_stride, void* q, int64_t q_stride, float* scales, int rows,
@@ -53,12 +54,12 @@ void launch_moe_align(const int* ids, int n, int expert_offset, int E_local, int
 void launch_grouped_gemm(int epilogue, const void* A, int64_t a_stride, const void* W, int64_t w_expert_stride,
                          const int* sorted_ids, const int* tile_expert, const int* meta, const float* topk_w, int top_k,
                          void* out, int64_t out_stride, int K, int N_out, int max_tiles, int k_splits, int64_t slab_elems,
-                         hipStream_t stream);
+                         hipStream_t stream, float act_limit = 0.f);
 // 256×256×64 tile (gemm256.hip): large-M grouped GEMM and dense GEMM with optional SwiGLU epilogue
 void launch_grouped_gemm256(int epilogue, const void* A, int64_t a_stride, const void* W, int64_t w_expert_stride,
                             const int* sorted_ids, const int* tile_expert, const int* meta, const float* topk_w, int top_k,
                             void* out, int64_t out_stride, int K, int N_out, int max_tiles, int k_splits, int64_t slab_elems,
-                            hipStream_t stream);
+                            hipStream_t stream, float act_limit = 0.f);
 void launch_dense_gemm256(bool swiglu, const void* x, int64_t x_stride, const void* W, void* out, int64_t out_stride, int M,
                           int K, int N_out, int k_splits, float* workspace, bool split_tail, hipStream_t stream);
 void dense_gemm256_tail_plan(int M, int K, int N_out, bool swiglu, int* tail_tiles, int* tail_slices);
@@ -195,12 +196,16 @@ void launch_rm_causal_conv(const void* x, bool bf16, int64_t x_stride, const flo
                            int rows, int seqs, int C, void* out, bool out_bf16, hipStream_t stream);
 void launch_rm_rglru_scan(const void* z, const void* u, const void* y, bool bf16, int64_t y_stride, const float* gate_bias,
                           const float* rate, float* state, const int* positions, const int* qsl, const int* state_slots,
-                          const int* counts, int rows, int seqs, int B, int n, void* out, bool out_bf16, hipStream_t stream);
+                          const int* counts, int rows, int seqs, int B, int n, void* out, bool out_bf16, const int* tile_seq,
+                          const int* tile_q0, int num_tiles, float* ws, hipStream_t stream);
+int64_t rm_rglru_ws_floats(int rows, int seqs, int C);
 void launch_rm_latent_norm_cache(const void* proj, bool bf16, int64_t p_stride, int Q, const float* qw, const float* cw, float eps,
                                  const int* positions, const double* freq, float mag, int rot_dims, const int* slot_mapping, void* cache,
                                  int rows, int C, int R, void* cq, hipStream_t stream);
 void launch_rm_rotate_heads(void* q, bool bf16, int64_t q_stride, const int* positions, const double* freq, float mag, int rot_dims,
                             int rows, int H, int D, int R, hipStream_t stream);
+void launch_rm_identity_add(void* out, const void* h, bool bf16, int64_t h_stride, const int* ids, const float* wts, int K, int E,
+                            int rows, int W, hipStream_t stream);
 void launch_rm_gate_heads(const void* o, const void* gate, bool bf16, int64_t g_stride, int H, int rows, int Dv, void* out,
                           hipStream_t stream);
 void launch_dm_relu2_rows(const void* x, bool bf16, int64_t x_stride, int rows, int F, void* out, hipStream_t stream);

@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(
     const uint16_t* __restrict__ W, int64_t w_expert_stride,  // [E_local, N_total, K]
     const int* __restrict__ sorted_ids, const int* __restrict__ tile_expert, const int* __restrict__ meta,
     const float* __restrict__ topk_w, int top_k, void* __restrict__ out_, int64_t out_stride, int K, int N_half,
-    int n_col_blocks, int k_splits, int64_t slab_elems) {
+    int n_col_blocks, int k_splits, int64_t slab_elems, float act_limit) {
   uint16_t* out = reinterpret_cast<uint16_t*>(out_);
   constexpr int STAGE = 2 * BM * BK * 2;                     // A tile + B tile of one K-step
   __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];   // double-buffered, filled by LDS-DMA
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float gate = acc[m][n][r], up = acc[m][n + 2][r];
-          o[r] = (short)f2bf(gate * fast_rcp(1.f + fast_exp2(-1.4426950408889634f * gate)) * up);
+          o[r] = (short)f2bf(gated_act(gate, up, act_limit));
         }
         *reinterpret_cast<bf16x4*>(dst + n * 16) = o;           // padding rows hold finite junk, never read back
       }
@@ -357,7 +357,7 @@ void launch_moe_align(const int* ids, int n, int expert_offset, int E_local, int
 void launch_grouped_gemm(int epilogue, const void* A, int64_t a_stride, const void* W, int64_t w_expert_stride,
                          const int* sorted_ids, const int* tile_expert, const int* meta, const float* topk_w, int top_k,
                          void* out, int64_t out_stride, int K, int N_out, int max_tiles, int k_splits, int64_t slab_elems,
-                         hipStream_t stream) {
+                         hipStream_t stream, float act_limit) {
   if (max_tiles == 0) return;
   const int n_col_blocks = N_out / (epilogue == EPI_SWIGLU ? BN / 2 : BN);
   const int n_virtual = n_col_blocks * k_splits;
@@ -366,7 +366,7 @@ void launch_grouped_gemm(int epilogue, const void* A, int64_t a_stride, const vo
 #define DLI_GG(EPI)                                                                                                       \
   hipLaunchKernelGGL(grouped_gemm_kernel<EPI>, grid, dim3(256), 0, stream, (const uint16_t*)A, a_stride, (const uint16_t*)W, \
                      w_expert_stride, sorted_ids, tile_expert, meta, topk_w, top_k, out, out_stride, K, N_out, n_col_blocks, \
-                     k_splits, slab_elems)
+                     k_splits, slab_elems, act_limit)
   if (epilogue == EPI_SWIGLU) DLI_GG(EPI_SWIGLU);
   else if (epilogue == EPI_RELU2) DLI_GG(EPI_RELU2);
   else if (epilogue == EPI_SCATTER) DLI_GG(EPI_SCATTER);

@@ -91,17 +91,41 @@ __global__ __launch_bounds__(NT) void conv_rows_kernel(const A* __restrict__ x, 
 //   r = sigmoid(z[b, t, j] + gb[c]),  i = sigmoid(z[b, t, n + j] + gb[C + c]),  log a = -rate[c] · r,
 //   S ← exp(log a) · S + sqrt(1 - exp(2 log a)) · i · u[t, c],   out[t, c] = S · gelu_tanh(y[t, c])
 // with S the sequence's state row (zero at position 0), written back after its last token of the step.  A thread owns one
-// channel of one sequence; the next token's operands are fetched while the current one is applied.
-template <typename A, typename O>
+// channel of one work item and fetches four tokens' operands at a time.
+//
+// A work item is either a whole sequence of the step (MODE 0: one-token rows — and every sequence when the step has no block
+// list) or one 64-token block of a longer chunk (three launches, so that the blocks of a long chunk run side by side):
+//   MODE 1  per block: Σ log a over the block and the block's own contribution L (state from zero, no output) → ws[block]
+//   prefix  per sequence (rglru_prefix_kernel): walks its blocks in order, leaves in ws[block] the state at the block's START
+//           and in the sequence's state slot the state after its last token: S ← exp(Σ log a) · S + L
+//   MODE 2  per block: the recurrence again from ws[block], now with outputs.
+// Blocks are the step's prefill tiles (tile_seq / tile_q0, 64 tokens); ws row of a block = (first token >> 6) + batch row
+// (unique: rows of later sequences start at later tokens); a ws row is [2][C] = (Σ log a | L, then the start state).
+template <typename A, typename O, int MODE>
 __global__ __launch_bounds__(NT) void rglru_scan_kernel(const A* __restrict__ z, const A* __restrict__ u, const A* __restrict__ y,
                                                         int64_t y_stride, const float* __restrict__ gb, const float* __restrict__ rate,
                                                         float* __restrict__ state, const int* __restrict__ positions,
                                                         const int* __restrict__ qsl, const int* __restrict__ state_slots,
-                                                        const int* __restrict__ counts, int T, int B, int n, O* __restrict__ out) {
-  const int seq = blockIdx.y;
-  if (seq >= counts[3]) return;
+                                                        const int* __restrict__ counts, int T, int B, int n, O* __restrict__ out,
+                                                        const int* __restrict__ tile_seq, const int* __restrict__ tile_q0,
+                                                        int num_tiles, float* __restrict__ ws, int single_only) {
+  int seq, t0, t1;
+  if (MODE == 0) {
+    seq = blockIdx.y;
+    if (seq >= counts[3]) return;
+    t0 = qsl[seq];
+    t1 = qsl[seq + 1];
+    if (single_only && t1 - t0 != 1) return;               // longer chunks take the block path
+  } else {
+    const int tile = blockIdx.y;
+    if (tile >= min(counts[2], num_tiles)) return;
+    seq = tile_seq[tile];
+    const int s0 = qsl[seq], s1 = qsl[seq + 1];
+    if (s1 - s0 < 2) return;                               // one-token rows belong to MODE 0
+    t0 = s0 + tile_q0[tile];
+    t1 = min(t0 + 64, s1);
+  }
   const int slot = state_slots[seq];
-  const int t0 = qsl[seq], t1 = qsl[seq + 1];
   if (slot < 0 || t1 <= t0) return;
   const int C = B * n;
   const int c = blockIdx.x * NT + threadIdx.x;
@@ -109,24 +133,59 @@ __global__ __launch_bounds__(NT) void rglru_scan_kernel(const A* __restrict__ z,
   const int b = c / n, j = c - b * n;
   const float br = gb[c], bi = gb[C + c], rt = rate[c];
   float* sp = state + (int64_t)slot * C + c;
-  float S = positions[t0] > 0 ? *sp : 0.f;
+  float* wr = ws + ((int64_t)((t0 >> 6) + seq) * 2) * C + c;
+  float S = MODE == 0 ? (positions[t0] > 0 ? *sp : 0.f) : (MODE == 2 ? wr[C] : 0.f);
+  float LA = 0.f;
   const A* zp = z + ((int64_t)b * T + t0) * 2 * n + j;
-  float zr = ldf<A>(zp), zi = ldf<A>(zp + n), uu = ldf<A>(u + (int64_t)t0 * C + c), yy = ldf<A>(y + (int64_t)t0 * y_stride + c);
-  for (int t = t0; t < t1; ++t) {
-    const float czr = zr, czi = zi, cu = uu, cy = yy;
-    if (t + 1 < t1) {
-      zp += 2 * n;
-      zr = ldf<A>(zp);
-      zi = ldf<A>(zp + n);
-      uu = ldf<A>(u + (int64_t)(t + 1) * C + c);
-      yy = ldf<A>(y + (int64_t)(t + 1) * y_stride + c);
+  for (int t = t0; t < t1; t += 4) {
+    float zr[4], zi[4], uu[4], yy[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const bool live = t + k < t1;
+      zr[k] = live ? ldf<A>(zp + (int64_t)k * 2 * n) : 0.f;
+      zi[k] = live ? ldf<A>(zp + (int64_t)k * 2 * n + n) : 0.f;
+      uu[k] = live ? ldf<A>(u + (int64_t)(t + k) * C + c) : 0.f;
+      yy[k] = (MODE != 1 && live) ? ldf<A>(y + (int64_t)(t + k) * y_stride + c) : 0.f;
     }
-    const float la = -rt * sigmoid_f(czr + br);
-    const float a = expf(la);
-    S = a * S + sqrtf(-expm1f(2.f * la)) * sigmoid_f(czi + bi) * cu;
-    stf<O>(out + (int64_t)t * C + c, S * gelu_tanh_f(cy));
+    zp += 8 * n;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (t + k < t1) {
+        const float la = -rt * sigmoid_f(zr[k] + br);
+        S = expf(la) * S + sqrtf(-expm1f(2.f * la)) * sigmoid_f(zi[k] + bi) * uu[k];
+        if (MODE == 1) LA += la;
+        else stf<O>(out + (int64_t)(t + k) * C + c, S * gelu_tanh_f(yy[k]));
+      }
+    }
   }
-  *sp = S;
+  if (MODE == 0) *sp = S;
+  if (MODE == 1) {
+    wr[0] = LA;
+    wr[C] = S;
+  }
+}
+
+// per (sequence with a chunk of two tokens or more, channel): see above
+__global__ __launch_bounds__(NT) void rglru_prefix_kernel(float* __restrict__ state, float* __restrict__ ws,
+                                                          const int* __restrict__ positions, const int* __restrict__ qsl,
+                                                          const int* __restrict__ state_slots, const int* __restrict__ counts, int C) {
+  const int seq = blockIdx.y;
+  if (seq >= counts[3]) return;
+  const int t0 = qsl[seq], nt = qsl[seq + 1] - t0;
+  const int slot = state_slots[seq];
+  if (slot < 0 || nt < 2) return;
+  const int c = blockIdx.x * NT + threadIdx.x;
+  if (c >= C) return;
+  float* sp = state + (int64_t)slot * C + c;
+  float run = positions[t0] > 0 ? *sp : 0.f;
+  const int blocks = (nt + 63) >> 6;
+  for (int i = 0; i < blocks; ++i) {
+    float* wr = ws + ((int64_t)(((t0 + 64 * i) >> 6) + seq) * 2) * C + c;
+    const float la = wr[0], own = wr[C];
+    wr[C] = run;
+    run = expf(la) * run + own;
+  }
+  *sp = run;
 }
 
 // ------------------------------------------------------------------------------------------------ latents: norms, rotation, cache
@@ -227,6 +286,21 @@ __global__ __launch_bounds__(NT) void gate_heads_kernel(const A* __restrict__ o,
   }
 }
 
+// out[t, :] += (Σ over the slots of token t whose id is not one of the E experts of wts[t, slot]) · h[t, :] — the identity
+// experts of a routed feed-forward whose real experts ran elsewhere
+template <typename A>
+__global__ __launch_bounds__(NT) void identity_add_kernel(A* __restrict__ out, const A* __restrict__ h, int64_t h_stride,
+                                                          const int* __restrict__ ids, const float* __restrict__ wts, int K, int E, int W) {
+  const int64_t t = blockIdx.x;
+  float idw = 0.f;
+  for (int k = 0; k < K; ++k) {
+    const int e = ids[t * K + k];
+    if (e < 0 || e >= E) idw += wts[t * K + k];
+  }
+  if (idw == 0.f) return;
+  for (int c = threadIdx.x; c < W; c += NT) stf<A>(out + t * W + c, ldf<A>(out + t * W + c) + idw * ldf<A>(h + t * h_stride + c));
+}
+
 }  // namespace
 
 // ================================================================================================ launchers
@@ -255,14 +329,27 @@ void launch_rm_causal_conv(const void* x, bool bf16, int64_t x_stride, const flo
                                         state_slots, counts, C));
 }
 
+int64_t rm_rglru_ws_floats(int rows, int seqs, int C) { return (int64_t)((rows >> 6) + seqs + 1) * 2 * C; }
+
 void launch_rm_rglru_scan(const void* z, const void* u, const void* y, bool bf16, int64_t y_stride, const float* gate_bias,
                           const float* rate, float* state, const int* positions, const int* qsl, const int* state_slots,
-                          const int* counts, int rows, int seqs, int B, int n, void* out, bool out_bf16, hipStream_t stream) {
+                          const int* counts, int rows, int seqs, int B, int n, void* out, bool out_bf16, const int* tile_seq,
+                          const int* tile_q0, int num_tiles, float* ws, hipStream_t stream) {
   if (rows == 0 || seqs == 0) return;
-  const dim3 grid((B * n + NT - 1) / NT, seqs);
-  RM_BF16(bf16, A, RM_BF16(out_bf16, O, hipLaunchKernelGGL((rglru_scan_kernel<A, O>), grid, dim3(NT), 0, stream, (const A*)z, (const A*)u,
-                                                           (const A*)y, y_stride, gate_bias, rate, state, positions, qsl, state_slots,
-                                                           counts, rows, B, n, (O*)out)));
+  const int C = B * n, cb = (C + NT - 1) / NT;
+  const bool blocks = num_tiles > 0 && ws != nullptr;
+#define RM_SCAN(MODE, grid_y)                                                                                                          \
+  RM_BF16(bf16, A, RM_BF16(out_bf16, O, hipLaunchKernelGGL((rglru_scan_kernel<A, O, MODE>), dim3(cb, grid_y), dim3(NT), 0, stream,     \
+                                                           (const A*)z, (const A*)u, (const A*)y, y_stride, gate_bias, rate, state,  \
+                                                           positions, qsl, state_slots, counts, rows, B, n, (O*)out, tile_seq,       \
+                                                           tile_q0, num_tiles, ws, blocks ? 1 : 0)))
+  RM_SCAN(0, seqs);
+  if (blocks) {
+    RM_SCAN(1, num_tiles);
+    hipLaunchKernelGGL(rglru_prefix_kernel, dim3(cb, seqs), dim3(NT), 0, stream, state, ws, positions, qsl, state_slots, counts, C);
+    RM_SCAN(2, num_tiles);
+  }
+#undef RM_SCAN
 }
 
 void launch_rm_latent_norm_cache(const void* proj, bool bf16, int64_t p_stride, int Q, const float* qw, const float* cw, float eps,
@@ -279,6 +366,13 @@ void launch_rm_rotate_heads(void* q, bool bf16, int64_t q_stride, const int* pos
   if (rows == 0 || rot_dims == 0) return;
   RM_BF16(bf16, A, hipLaunchKernelGGL(rotate_heads_kernel<A>, dim3(rows), dim3(NT), rot_dims * sizeof(float), stream, (A*)q, q_stride,
                                       positions, freq, mag, rot_dims, H, D, R));
+}
+
+void launch_rm_identity_add(void* out, const void* h, bool bf16, int64_t h_stride, const int* ids, const float* wts, int K, int E,
+                            int rows, int W, hipStream_t stream) {
+  if (rows == 0) return;
+  RM_BF16(bf16, A, hipLaunchKernelGGL(identity_add_kernel<A>, dim3(rows), dim3(NT), 0, stream, (A*)out, (const A*)h, h_stride, ids, wts,
+                                      K, E, W));
 }
 
 void launch_rm_gate_heads(const void* o, const void* gate, bool bf16, int64_t g_stride, int H, int rows, int Dv, void* out,

@@ -37,7 +37,7 @@ Tensor rm_causal_conv(const Tensor& x, const Tensor& w, const c10::optional<Tens
 // state fp32 [slots, B·n] → S · gelu_tanh(y), rows of padding zero
 Tensor rm_rglru_scan(const Tensor& z, const Tensor& u, const Tensor& y, const Tensor& gate_bias, const Tensor& rate, Tensor state,
                      const Tensor& positions, const Tensor& qsl, const Tensor& state_slots, const Tensor& counts, int64_t num_seqs,
-                     bool out_bf16) {
+                     bool out_bf16, const c10::optional<Tensor>& tile_seq, const c10::optional<Tensor>& tile_q0, int64_t num_tiles) {
   const bool bf = act_bf16(u, "u");
   check_act_like(z, bf, "z");
   check_act_like(y, bf, "y");
@@ -52,9 +52,24 @@ Tensor rm_rglru_scan(const Tensor& z, const Tensor& u, const Tensor& y, const Te
   TORCH_CHECK(state.dim() == 2 && state.size(1) == C, "state must be [slots, B·n]");
   check_step_meta(positions, qsl, state_slots, counts, T, num_seqs);
   Tensor out = at::zeros({T, C}, u.options().dtype(out_bf16 ? at::kBFloat16 : at::kFloat));
+  // chunks of two tokens or more run block-parallel over the step's 64-token tiles when the caller hands them in
+  const int* tsp = nullptr;
+  const int* tqp = nullptr;
+  Tensor ws;
+  if (num_tiles > 0 && tile_seq.has_value() && tile_q0.has_value()) {
+    check_i32(*tile_seq, "tile_seq");
+    check_i32(*tile_q0, "tile_q0");
+    TORCH_CHECK(tile_seq->numel() >= num_tiles && tile_q0->numel() >= num_tiles, "tile lists shorter than num_tiles");
+    tsp = tile_seq->data_ptr<int>();
+    tqp = tile_q0->data_ptr<int>();
+    ws = at::empty({dli::rm_rglru_ws_floats((int)T, (int)num_seqs, (int)C)}, u.options().dtype(at::kFloat));
+  } else {
+    num_tiles = 0;
+  }
   dli::launch_rm_rglru_scan(z.data_ptr(), u.data_ptr(), y.data_ptr(), bf, y.stride(0), gate_bias.data_ptr<float>(), rate.data_ptr<float>(),
                             state.data_ptr<float>(), positions.data_ptr<int>(), qsl.data_ptr<int>(), state_slots.data_ptr<int>(),
-                            counts.data_ptr<int>(), (int)T, (int)num_seqs, (int)B, (int)n, out.data_ptr(), out_bf16, cur_stream(u));
+                            counts.data_ptr<int>(), (int)T, (int)num_seqs, (int)B, (int)n, out.data_ptr(), out_bf16, tsp, tqp, (int)num_tiles,
+                            num_tiles > 0 ? ws.data_ptr<float>() : nullptr, cur_stream(u));
   return out;
 }
 
@@ -137,8 +152,17 @@ Tensor rm_clamped_experts(const Tensor& h, const Tensor& ids, const Tensor& wts,
   check_f32(wts, "wts");
   TORCH_CHECK(ids.dim() == 2 && ids.size(0) == T && wts.dim() == 2 && wts.size(0) == T && wts.size(1) == ids.size(1), "ids / wts must be [T, K]");
   const int64_t K = ids.size(1);
-  TORCH_CHECK(W * 4 <= kSmMaxLds && K * F * 4 <= kSmMaxLds, "rows too wide");
   Tensor out = at::empty({T, W}, h.options());
+  if (bf && g_dm_grouped_experts && W % 128 == 0 && F % 64 == 0 && E <= 64 && (T * K >= 64 || F % 128 == 0) && h.is_contiguous() &&
+      reinterpret_cast<uintptr_t>(h.data_ptr()) % 16 == 0) {
+    // the expert kernels of the Mixtral path (weight streaming at decode size, else grouped GEMMs) with the clamped activation
+    // in their first epilogue; pairs of identity experts are outside the expert range and skipped there
+    moe_apply(h, ids, wts, gate_up, down, K, 0, E, 0, out, cur_stream(h), (float)limit);
+    dli::launch_rm_identity_add(out.data_ptr(), h.data_ptr(), bf, h.stride(0), ids.data_ptr<int>(), wts.data_ptr<float>(), (int)K, (int)E,
+                                (int)T, (int)W, cur_stream(h));
+    return out;
+  }
+  TORCH_CHECK(W * 4 <= kSmMaxLds && K * F * 4 <= kSmMaxLds, "rows too wide");
   Tensor act = at::empty({T * K, F}, h.options());
   dli::launch_dm_experts(h.data_ptr(), bf, h.stride(0), ids.data_ptr<int>(), wts.data_ptr<float>(), (int)K, gate_up.data_ptr(),
                          down.data_ptr(), (int)T, (int)F, (int)W, act.data_ptr(), out.data_ptr(), 2, (int)E, (float)limit, cur_stream(h));

@@ -338,7 +338,7 @@ const int64_t g_moe_skinny_max_t = std::getenv("DLI_NO_SKINNY_MOE") ? 0
 // slot) pairs whose expert ids / gate weights are already on the device (``ids`` < 0 or outside the local range: skipped).
 // ``out``: [T, H] bf16 (any device memory: the expert-parallel path hands in its IPC-visible result buffer).
 void moe_experts_forward(const Tensor& x, const Tensor& ids, const Tensor& wts, const Tensor& w13, const Tensor& w2, int64_t top_k,
-                         int64_t expert_offset, bool big, void* out, hipStream_t stream) {
+                         int64_t expert_offset, bool big, void* out, hipStream_t stream, float act_limit = 0.f) {
   const int64_t T = x.size(0), H = x.size(1), El = w13.size(0), I = w13.size(1) / 2;
   const int64_t n = T * top_k;
   auto i32 = x.options().dtype(at::kInt);
@@ -362,10 +362,10 @@ void moe_experts_forward(const Tensor& x, const Tensor& ids, const Tensor& wts, 
                         tile_expert.data_ptr<int>(), meta.data_ptr<int>(), (int)capacity, (int)TR, stream);
   auto gg = big ? dli::launch_grouped_gemm256 : dli::launch_grouped_gemm;
   gg(0, x.data_ptr(), H, w13.data_ptr(), 2 * I * H, sorted.data_ptr<int>(), tile_expert.data_ptr<int>(), meta.data_ptr<int>(),
-     wts.data_ptr<float>(), (int)top_k, act.data_ptr(), I, (int)H, (int)I, (int)max_tiles, 1, 0, stream);
+     wts.data_ptr<float>(), (int)top_k, act.data_ptr(), I, (int)H, (int)I, (int)max_tiles, 1, 0, stream, act_limit);
   gg(split ? 2 : 1, act.data_ptr(), I, w2.data_ptr(), H * I, sorted.data_ptr<int>(), tile_expert.data_ptr<int>(),
      meta.data_ptr<int>(), wts.data_ptr<float>(), (int)top_k, y.data_ptr(), H, (int)I, (int)H, (int)max_tiles, (int)k_splits,
-     n * H, stream);
+     n * H, stream, 0.f);
   dli::launch_moe_sum(y.data_ptr(), split, (int)k_splits, n * H, ids.data_ptr<int>(), (int)expert_offset, (int)El, (int)top_k,
                       (int)T, (int)H, out, stream);
 }
@@ -373,7 +373,7 @@ void moe_experts_forward(const Tensor& x, const Tensor& ids, const Tensor& wts, 
 // ---- experts of tokens whose (expert id, weight) pairs are already on the device: the decode-sized weight-streaming path or
 // the grouped GEMMs, chosen as for the Mixtral block (tile_rows: 0 = by the row count, 128 / 256 = forced)
 void moe_apply(const Tensor& x, const Tensor& ids, const Tensor& wts, const Tensor& w13, const Tensor& w2, int64_t top_k,
-               int64_t expert_offset, int64_t E, int64_t tile_rows, Tensor& out, hipStream_t stream) {
+               int64_t expert_offset, int64_t E, int64_t tile_rows, Tensor& out, hipStream_t stream, float act_limit = 0.f) {
   const int64_t T = x.size(0), H = x.size(1), El = w13.size(0), I = w13.size(1) / 2;
   auto i32 = x.options().dtype(at::kInt);
   const int64_t n = T * top_k;
@@ -396,7 +396,7 @@ void moe_apply(const Tensor& x, const Tensor& ids, const Tensor& wts, const Tens
     dli::launch_moe_skinny(false, x.data_ptr(), H, w13.data_ptr(), 2 * I * H, sorted.data_ptr<int>(), tile_expert.data_ptr<int>(),
                            meta.data_ptr<int>(), wts.data_ptr<float>(), (int)top_k, gu.data_ptr(), 2 * I, (int)H, (int)(2 * I),
                            (int)tiles, (int)T, stream);
-    dli::launch_silu_and_mul(act16.data_ptr(), gu.data_ptr(), (int)(tiles * rows_pad), (int)I, 2 * I, stream);
+    dli::launch_silu_and_mul(act16.data_ptr(), gu.data_ptr(), (int)(tiles * rows_pad), (int)I, 2 * I, stream, act_limit);
     dli::launch_moe_skinny(true, act16.data_ptr(), I, w2.data_ptr(), H * I, sorted.data_ptr<int>(), tile_expert.data_ptr<int>(),
                            meta.data_ptr<int>(), wts.data_ptr<float>(), (int)top_k, y16.data_ptr(), H, (int)I, (int)H,
                            (int)tiles, (int)T, stream);
@@ -404,7 +404,7 @@ void moe_apply(const Tensor& x, const Tensor& ids, const Tensor& wts, const Tens
                         (int)H, out.data_ptr(), stream);
     return;
   }
-  moe_experts_forward(x, ids, wts, w13, w2, top_k, expert_offset, big, out.data_ptr(), stream);
+  moe_experts_forward(x, ids, wts, w13, w2, top_k, expert_offset, big, out.data_ptr(), stream, act_limit);
 }
 
 // ---- MoE: route → align → grouped GEMM (SwiGLU epilogue) → grouped GEMM (weighted scatter) → sum ----
@@ -641,7 +641,8 @@ TORCH_LIBRARY(dli, m) {
   m.def("rm_causal_conv(Tensor x, Tensor w, Tensor? bias, Tensor(a!) state, Tensor positions, Tensor token_seq, Tensor qsl, "
         "Tensor state_slots, Tensor counts, int num_seqs, bool out_bf16) -> Tensor", &rm_causal_conv);
   m.def("rm_rglru_scan(Tensor z, Tensor u, Tensor y, Tensor gate_bias, Tensor rate, Tensor(a!) state, Tensor positions, Tensor qsl, "
-        "Tensor state_slots, Tensor counts, int num_seqs, bool out_bf16) -> Tensor", &rm_rglru_scan);
+        "Tensor state_slots, Tensor counts, int num_seqs, bool out_bf16, Tensor? tile_seq=None, Tensor? tile_q0=None, int num_tiles=0) "
+        "-> Tensor", &rm_rglru_scan);
   m.def("rm_latent_norm_cache(Tensor proj, int Q, Tensor qw, Tensor? cw, float eps, Tensor positions, Tensor freq, float mag, "
         "int rot_dims, Tensor slot_mapping, Tensor(a!)? cache, int C, int R) -> Tensor", &rm_latent_norm_cache);
   m.def("rm_rotate_heads(Tensor(a!) q, Tensor positions, Tensor freq, float mag, int rot_dims, int H, int D, int R) -> ()",

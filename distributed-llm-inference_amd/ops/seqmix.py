@@ -702,8 +702,11 @@ def rglru_scan(z: torch.Tensor, u: torch.Tensor, y: torch.Tensor, gate_bias: tor
     ``a = exp(-rate · sigmoid(z_r + b_r))``, ``S ← a · S + sqrt(1 - a²) · sigmoid(z_i + b_i) · u`` with ``S`` the sequence's
     ``state[slot]`` row (zero at position 0), written back after the step's last token.  Returns ``S · gelu_tanh(y)``."""
     if _act_ok(u):
+        # chunks run block-parallel over the step's 64-token tiles (local states → prefix over blocks → outputs)
+        tiles = meta.num_prefill_tiles if BLOCK_SCAN else 0
         return _hip().rm_rglru_scan(z, u, y, gate_bias, rate, state, meta.positions, meta.query_start_loc, meta.state_slots,
-                                    meta.counts, meta.num_seqs, out_dtype == torch.bfloat16)
+                                    meta.counts, meta.num_seqs, out_dtype == torch.bfloat16, meta.prefill_tile_seq if tiles else None,
+                                    meta.prefill_tile_q0 if tiles else None, tiles)
     B, T, n2 = z.shape
     n = n2 // 2
     zf = z.float().view(B, T, 2, n).permute(2, 1, 0, 3).reshape(2, T, B * n)
