@@ -29,17 +29,56 @@ template <typename A> __device__ __forceinline__ void stf(A* p, float v);
 template <> __device__ __forceinline__ void stf<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void stf<uint16_t>(uint16_t* p, float v) { *p = f2bf(v); }
 
-__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
-__device__ __forceinline__ float gelu_tanh_f(float z) {
-  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+// sigmoid, exp and the tanh-form GELU on the hardware's exp2 / reciprocal (about one ulp each); 0.5 · (1 + tanh v) = sigmoid(2v)
+__device__ __forceinline__ float sigmoid_f(float z) { return fast_rcp(1.f + fast_exp2(-1.4426950408889634f * z)); }
+__device__ __forceinline__ float exp_f(float z) { return fast_exp2(1.4426950408889634f * z); }
+__device__ __forceinline__ float gelu_tanh_f(float z) { return z * sigmoid_f(1.5957691216057308f * (z + 0.044715f * z * z * z)); }
+// 1 − exp(x) for x ≤ 0 without the cancellation near zero (three terms of the series below 0.1: relative error < 5e-6 · x)
+__device__ __forceinline__ float one_minus_exp(float x) {
+  return x > -0.1f ? -x * (1.f + x * (0.5f + x * (0.16666667f + x * 0.041666668f))) : 1.f - exp_f(x);
 }
+
+// V consecutive row elements ↔ fp32: V = 4 takes 16-byte / 8-byte accesses (the launchers check divisibility and alignment)
+template <typename A, int V> struct Vec {
+  float v[V];
+  __device__ __forceinline__ void load(const A* p) {
+    if constexpr (V == 4) {
+      if constexpr (sizeof(A) == 4) {
+        const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+        v[0] = t[0]; v[1] = t[1]; v[2] = t[2]; v[3] = t[3];
+      } else {
+        const bf16x4 t = *reinterpret_cast<const bf16x4*>(p);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = bf2f((uint16_t)t[j]);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < V; ++j) v[j] = ldf<A>(p + j);
+    }
+  }
+  __device__ __forceinline__ void store(A* p) const {
+    if constexpr (V == 4) {
+      if constexpr (sizeof(A) == 4) {
+        *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
+      } else {
+        bf16x4 t;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t[j] = (short)f2bf(v[j]);
+        *reinterpret_cast<bf16x4*>(p) = t;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < V; ++j) stf<A>(p + j, v[j]);
+    }
+  }
+};
 
 // ------------------------------------------------------------------------------------------------ convolution
 // out[t, c] = bias[c] + Σ_j w[j, c] · x[t - taps + 1 + j, c] over the rows of the token's own sequence: rows of this step's
 // chunk, the sequence's state rows (its last taps-1 inputs, oldest first: positions p0-taps+1 … p0-1 for a chunk starting at
 // p0) before the chunk, nothing before position 0 (so a reused slot needs no clearing).  One workgroup per token; a thread
 // keeps one channel per trip, so all taps of a channel are coalesced row reads.
-template <typename A, typename O>
+template <typename A, typename O, int V>
 __global__ __launch_bounds__(NT) void causal_conv_kernel(const A* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
                                                          const float* __restrict__ bias, int taps, const float* __restrict__ state,
                                                          const int* __restrict__ positions, const int* __restrict__ token_seq,
@@ -55,14 +94,32 @@ __global__ __launch_bounds__(NT) void causal_conv_kernel(const A* __restrict__ x
   const int back = (int)t - qsl[seq];                             // rows of the chunk above this one
   const float* st = state + (int64_t)state_slots[seq] * (taps - 1) * C;
   const A* xr = x + t * x_stride;
-  for (int c = threadIdx.x; c < C; c += NT) {
-    float a = bias != nullptr ? bias[c] : 0.f;
+  for (int c = threadIdx.x * V; c < C; c += NT * V) {
+    Vec<float, V> a;
+    if (bias != nullptr) a.load(bias + c);
+    else
+#pragma unroll
+      for (int k = 0; k < V; ++k) a.v[k] = 0.f;
+#pragma unroll 4
     for (int j = max(taps - 1 - p, 0); j < taps; ++j) {           // taps that would reach before position 0 are skipped
       const int d = taps - 1 - j;                                  // how far back the tap reaches
-      const float v = d <= back ? ldf<A>(xr - (int64_t)d * x_stride + c) : st[(int64_t)(taps - 1 - (d - back)) * C + c];
-      a += w[(int64_t)j * C + c] * v;
+      Vec<float, V> v, wj;
+      if (d <= back) {
+        Vec<A, V> xv;
+        xv.load(xr - (int64_t)d * x_stride + c);
+#pragma unroll
+        for (int k = 0; k < V; ++k) v.v[k] = xv.v[k];
+      } else {
+        v.load(st + (int64_t)(taps - 1 - (d - back)) * C + c);
+      }
+      wj.load(w + (int64_t)j * C + c);
+#pragma unroll
+      for (int k = 0; k < V; ++k) a.v[k] += wj.v[k] * v.v[k];
     }
-    stf<O>(out + t * C + c, a);
+    Vec<O, V> o;
+#pragma unroll
+    for (int k = 0; k < V; ++k) o.v[k] = a.v[k];
+    o.store(out + t * C + c);
   }
 }
 
@@ -152,7 +209,7 @@ __global__ __launch_bounds__(NT) void rglru_scan_kernel(const A* __restrict__ z,
     for (int k = 0; k < 4; ++k) {
       if (t + k < t1) {
         const float la = -rt * sigmoid_f(zr[k] + br);
-        S = expf(la) * S + sqrtf(-expm1f(2.f * la)) * sigmoid_f(zi[k] + bi) * uu[k];
+        S = exp_f(la) * S + sqrtf(one_minus_exp(2.f * la)) * sigmoid_f(zi[k] + bi) * uu[k];
         if (MODE == 1) LA += la;
         else stf<O>(out + (int64_t)(t + k) * C + c, S * gelu_tanh_f(yy[k]));
       }
@@ -183,7 +240,7 @@ __global__ __launch_bounds__(NT) void rglru_prefix_kernel(float* __restrict__ st
     float* wr = ws + ((int64_t)(((t0 + 64 * i) >> 6) + seq) * 2) * C + c;
     const float la = wr[0], own = wr[C];
     wr[C] = run;
-    run = expf(la) * run + own;
+    run = exp_f(la) * run + own;
   }
   *sp = run;
 }
@@ -273,22 +330,27 @@ __global__ __launch_bounds__(NT) void rotate_heads_kernel(A* __restrict__ q, int
   }
 }
 
-// out[t, h·Dv + d] = o[h, t, d] · sigmoid(gate[t, h·Dv + d])
-template <typename A>
+// out[t, h·Dv + d] = o[h, t, d] · sigmoid(gate[t, h·Dv + d]); V entries of a head per thread and trip
+template <typename A, int V>
 __global__ __launch_bounds__(NT) void gate_heads_kernel(const A* __restrict__ o, const A* __restrict__ gate, int64_t g_stride, int H,
                                                         int T, int Dv, A* __restrict__ out) {
   const int64_t n = (int64_t)T * H * Dv;
-  for (int64_t i = (int64_t)blockIdx.x * NT + threadIdx.x; i < n; i += (int64_t)gridDim.x * NT) {
+  for (int64_t i = ((int64_t)blockIdx.x * NT + threadIdx.x) * V; i < n; i += (int64_t)gridDim.x * NT * V) {
     const int64_t t = i / (H * Dv);
     const int r = (int)(i - t * (H * Dv));
     const int h = r / Dv, d = r - h * Dv;
-    stf<A>(out + i, ldf<A>(o + ((int64_t)h * T + t) * Dv + d) * sigmoid_f(ldf<A>(gate + t * g_stride + r)));
+    Vec<A, V> ov, gv, res;
+    ov.load(o + ((int64_t)h * T + t) * Dv + d);
+    gv.load(gate + t * g_stride + r);
+#pragma unroll
+    for (int k = 0; k < V; ++k) res.v[k] = ov.v[k] * sigmoid_f(gv.v[k]);
+    res.store(out + i);
   }
 }
 
 // out[t, :] += (Σ over the slots of token t whose id is not one of the E experts of wts[t, slot]) · h[t, :] — the identity
 // experts of a routed feed-forward whose real experts ran elsewhere
-template <typename A>
+template <typename A, int V>
 __global__ __launch_bounds__(NT) void identity_add_kernel(A* __restrict__ out, const A* __restrict__ h, int64_t h_stride,
                                                           const int* __restrict__ ids, const float* __restrict__ wts, int K, int E, int W) {
   const int64_t t = blockIdx.x;
@@ -298,7 +360,14 @@ __global__ __launch_bounds__(NT) void identity_add_kernel(A* __restrict__ out, c
     if (e < 0 || e >= E) idw += wts[t * K + k];
   }
   if (idw == 0.f) return;
-  for (int c = threadIdx.x; c < W; c += NT) stf<A>(out + t * W + c, ldf<A>(out + t * W + c) + idw * ldf<A>(h + t * h_stride + c));
+  for (int c = threadIdx.x * V; c < W; c += NT * V) {
+    Vec<A, V> ov, hv;
+    ov.load(out + t * W + c);
+    hv.load(h + t * h_stride + c);
+#pragma unroll
+    for (int k = 0; k < V; ++k) ov.v[k] += idw * hv.v[k];
+    ov.store(out + t * W + c);
+  }
 }
 
 }  // namespace
@@ -317,13 +386,20 @@ __global__ __launch_bounds__(NT) void identity_add_kernel(A* __restrict__ out, c
 
 int rm_max_taps() { return RM_MAX_TAPS; }
 
+static bool al16(const void* p) { return p == nullptr || reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
 void launch_rm_causal_conv(const void* x, bool bf16, int64_t x_stride, const float* w, const float* bias, int taps, float* state,
                            const int* positions, const int* token_seq, const int* qsl, const int* state_slots, const int* counts,
                            int rows, int seqs, int C, void* out, bool out_bf16, hipStream_t stream) {
   if (rows == 0) return;
-  RM_BF16(bf16, A, RM_BF16(out_bf16, O, hipLaunchKernelGGL((causal_conv_kernel<A, O>), dim3(rows), dim3(NT), 0, stream, (const A*)x,
-                                                           x_stride, w, bias, taps, state, positions, token_seq, qsl, state_slots, C,
-                                                           (O*)out)));
+  if (C % 4 == 0 && x_stride % 4 == 0 && al16(x) && al16(w) && al16(bias) && al16(state) && al16(out))
+    RM_BF16(bf16, A, RM_BF16(out_bf16, O, hipLaunchKernelGGL((causal_conv_kernel<A, O, 4>), dim3(rows), dim3(NT), 0, stream, (const A*)x,
+                                                             x_stride, w, bias, taps, state, positions, token_seq, qsl, state_slots, C,
+                                                             (O*)out)));
+  else
+    RM_BF16(bf16, A, RM_BF16(out_bf16, O, hipLaunchKernelGGL((causal_conv_kernel<A, O, 1>), dim3(rows), dim3(NT), 0, stream, (const A*)x,
+                                                             x_stride, w, bias, taps, state, positions, token_seq, qsl, state_slots, C,
+                                                             (O*)out)));
   if (taps > 1 && seqs > 0)
     RM_BF16(bf16, A, hipLaunchKernelGGL(conv_rows_kernel<A>, dim3(seqs), dim3(NT), 0, stream, (const A*)x, x_stride, taps, state, qsl,
                                         state_slots, counts, C));
@@ -371,17 +447,27 @@ void launch_rm_rotate_heads(void* q, bool bf16, int64_t q_stride, const int* pos
 void launch_rm_identity_add(void* out, const void* h, bool bf16, int64_t h_stride, const int* ids, const float* wts, int K, int E,
                             int rows, int W, hipStream_t stream) {
   if (rows == 0) return;
-  RM_BF16(bf16, A, hipLaunchKernelGGL(identity_add_kernel<A>, dim3(rows), dim3(NT), 0, stream, (A*)out, (const A*)h, h_stride, ids, wts,
-                                      K, E, W));
+  if (W % 4 == 0 && h_stride % 4 == 0 && al16(out) && al16(h))
+    RM_BF16(bf16, A, hipLaunchKernelGGL((identity_add_kernel<A, 4>), dim3(rows), dim3(NT), 0, stream, (A*)out, (const A*)h, h_stride, ids,
+                                        wts, K, E, W));
+  else
+    RM_BF16(bf16, A, hipLaunchKernelGGL((identity_add_kernel<A, 1>), dim3(rows), dim3(NT), 0, stream, (A*)out, (const A*)h, h_stride, ids,
+                                        wts, K, E, W));
 }
 
 void launch_rm_gate_heads(const void* o, const void* gate, bool bf16, int64_t g_stride, int H, int rows, int Dv, void* out,
                           hipStream_t stream) {
   const int64_t n = (int64_t)rows * H * Dv;
   if (n == 0) return;
-  const int blocks = (int)std::min<int64_t>((n + NT - 1) / NT, 16384);
-  RM_BF16(bf16, A, hipLaunchKernelGGL(gate_heads_kernel<A>, dim3(blocks), dim3(NT), 0, stream, (const A*)o, (const A*)gate, g_stride, H,
-                                      rows, Dv, (A*)out));
+  const bool wide = Dv % 4 == 0 && g_stride % 4 == 0 && al16(o) && al16(gate) && al16(out);
+  const int64_t items = wide ? n / 4 : n;
+  const int blocks = (int)std::min<int64_t>((items + NT - 1) / NT, 16384);
+  if (wide)
+    RM_BF16(bf16, A, hipLaunchKernelGGL((gate_heads_kernel<A, 4>), dim3(blocks), dim3(NT), 0, stream, (const A*)o, (const A*)gate, g_stride,
+                                        H, rows, Dv, (A*)out));
+  else
+    RM_BF16(bf16, A, hipLaunchKernelGGL((gate_heads_kernel<A, 1>), dim3(blocks), dim3(NT), 0, stream, (const A*)o, (const A*)gate, g_stride,
+                                        H, rows, Dv, (A*)out));
 }
 
 }  // namespace dli
