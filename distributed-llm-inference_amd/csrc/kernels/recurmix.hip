@@ -147,41 +147,31 @@ __global__ __launch_bounds__(NT) void conv_rows_kernel(const A* __restrict__ x, 
 // Per (sequence of the step, channel c = b·n + j), token by token in fp32:
 //   r = sigmoid(z[b, t, j] + gb[c]),  i = sigmoid(z[b, t, n + j] + gb[C + c]),  log a = -rate[c] · r,
 //   S ← exp(log a) · S + sqrt(1 - exp(2 log a)) · i · u[t, c],   out[t, c] = S · gelu_tanh(y[t, c])
-// with S the sequence's state row (zero at position 0), written back after its last token of the step.  A thread owns one
-// channel of one work item and fetches four tokens' operands at a time.
+// with S the sequence's state row (zero at position 0), written back after its last token of the step.
 //
-// A work item is either a whole sequence of the step (MODE 0: one-token rows — and every sequence when the step has no block
-// list) or one 64-token block of a longer chunk (three launches, so that the blocks of a long chunk run side by side):
-//   MODE 1  per block: Σ log a over the block and the block's own contribution L (state from zero, no output) → ws[block]
+// A work item is either a whole sequence of the step (rglru_scan_kernel: one-token rows — and every sequence when the step
+// has no block list) or one 64-token block of a longer chunk (three launches, so that the blocks of a long chunk run side by
+// side instead of one after the other):
+//   MODE 1  per block (rglru_block_kernel): Σ log a over the block and the block's own contribution L (state from zero, no
+//           output) → ws[block]
 //   prefix  per sequence (rglru_prefix_kernel): walks its blocks in order, leaves in ws[block] the state at the block's START
 //           and in the sequence's state slot the state after its last token: S ← exp(Σ log a) · S + L
 //   MODE 2  per block: the recurrence again from ws[block], now with outputs.
 // Blocks are the step's prefill tiles (tile_seq / tile_q0, 64 tokens); ws row of a block = (first token >> 6) + batch row
 // (unique: rows of later sequences start at later tokens); a ws row is [2][C] = (Σ log a | L, then the start state).
-template <typename A, typename O, int MODE>
+//
+// Whole sequences: a thread owns one channel of one sequence and fetches four tokens' operands at a time.
+template <typename A, typename O>
 __global__ __launch_bounds__(NT) void rglru_scan_kernel(const A* __restrict__ z, const A* __restrict__ u, const A* __restrict__ y,
                                                         int64_t y_stride, const float* __restrict__ gb, const float* __restrict__ rate,
                                                         float* __restrict__ state, const int* __restrict__ positions,
                                                         const int* __restrict__ qsl, const int* __restrict__ state_slots,
                                                         const int* __restrict__ counts, int T, int B, int n, O* __restrict__ out,
-                                                        const int* __restrict__ tile_seq, const int* __restrict__ tile_q0,
-                                                        int num_tiles, float* __restrict__ ws, int single_only) {
-  int seq, t0, t1;
-  if (MODE == 0) {
-    seq = blockIdx.y;
-    if (seq >= counts[3]) return;
-    t0 = qsl[seq];
-    t1 = qsl[seq + 1];
-    if (single_only && t1 - t0 != 1) return;               // longer chunks take the block path
-  } else {
-    const int tile = blockIdx.y;
-    if (tile >= min(counts[2], num_tiles)) return;
-    seq = tile_seq[tile];
-    const int s0 = qsl[seq], s1 = qsl[seq + 1];
-    if (s1 - s0 < 2) return;                               // one-token rows belong to MODE 0
-    t0 = s0 + tile_q0[tile];
-    t1 = min(t0 + 64, s1);
-  }
+                                                        int single_only) {
+  const int seq = blockIdx.y;
+  if (seq >= counts[3]) return;
+  const int t0 = qsl[seq], t1 = qsl[seq + 1];
+  if (single_only && t1 - t0 != 1) return;                 // longer chunks take the block path
   const int slot = state_slots[seq];
   if (slot < 0 || t1 <= t0) return;
   const int C = B * n;
@@ -190,9 +180,7 @@ __global__ __launch_bounds__(NT) void rglru_scan_kernel(const A* __restrict__ z,
   const int b = c / n, j = c - b * n;
   const float br = gb[c], bi = gb[C + c], rt = rate[c];
   float* sp = state + (int64_t)slot * C + c;
-  float* wr = ws + ((int64_t)((t0 >> 6) + seq) * 2) * C + c;
-  float S = MODE == 0 ? (positions[t0] > 0 ? *sp : 0.f) : (MODE == 2 ? wr[C] : 0.f);
-  float LA = 0.f;
+  float S = positions[t0] > 0 ? *sp : 0.f;
   const A* zp = z + ((int64_t)b * T + t0) * 2 * n + j;
   for (int t = t0; t < t1; t += 4) {
     float zr[4], zi[4], uu[4], yy[4];
@@ -202,7 +190,7 @@ __global__ __launch_bounds__(NT) void rglru_scan_kernel(const A* __restrict__ z,
       zr[k] = live ? ldf<A>(zp + (int64_t)k * 2 * n) : 0.f;
       zi[k] = live ? ldf<A>(zp + (int64_t)k * 2 * n + n) : 0.f;
       uu[k] = live ? ldf<A>(u + (int64_t)(t + k) * C + c) : 0.f;
-      yy[k] = (MODE != 1 && live) ? ldf<A>(y + (int64_t)(t + k) * y_stride + c) : 0.f;
+      yy[k] = live ? ldf<A>(y + (int64_t)(t + k) * y_stride + c) : 0.f;
     }
     zp += 8 * n;
 #pragma unroll
@@ -210,15 +198,94 @@ __global__ __launch_bounds__(NT) void rglru_scan_kernel(const A* __restrict__ z,
       if (t + k < t1) {
         const float la = -rt * sigmoid_f(zr[k] + br);
         S = exp_f(la) * S + sqrtf(one_minus_exp(2.f * la)) * sigmoid_f(zi[k] + bi) * uu[k];
-        if (MODE == 1) LA += la;
-        else stf<O>(out + (int64_t)(t + k) * C + c, S * gelu_tanh_f(yy[k]));
+        stf<O>(out + (int64_t)(t + k) * C + c, S * gelu_tanh_f(yy[k]));
       }
     }
   }
-  if (MODE == 0) *sp = S;
+  *sp = S;
+}
+
+// MODE 1 / MODE 2 of a 64-token block on a workgroup of four waves over 64 channels: wave w takes the block's tokens
+// 16w … 16w+15 — every operand of a wave's tokens is in flight at once, and the sequential chain is 16 steps, not 64.  Each
+// wave computes its tokens' decays and inputs once (kept in registers), leaves (Σ log a, own contribution) of its quarter in
+// LDS, and either wave 0 combines the four into the block's summary (MODE 1) or every wave starts from the block's start
+// state advanced over the quarters before its own and writes its outputs (MODE 2).
+template <typename A, typename O, int MODE>
+__global__ __launch_bounds__(NT) void rglru_block_kernel(const A* __restrict__ z, const A* __restrict__ u, const A* __restrict__ y,
+                                                         int64_t y_stride, const float* __restrict__ gb, const float* __restrict__ rate,
+                                                         const int* __restrict__ qsl, const int* __restrict__ state_slots,
+                                                         const int* __restrict__ counts, int T, int B, int n, O* __restrict__ out,
+                                                         const int* __restrict__ tile_seq, const int* __restrict__ tile_q0,
+                                                         int num_tiles, float* __restrict__ ws) {
+  __shared__ float sLA[4][64], sL[4][64];
+  const int tile = blockIdx.y;
+  if (tile >= min(counts[2], num_tiles)) return;
+  const int seq = tile_seq[tile];
+  const int s0 = qsl[seq], s1 = qsl[seq + 1];
+  if (s1 - s0 < 2 || state_slots[seq] < 0) return;           // one-token rows belong to the per-sequence kernel
+  const int t0 = s0 + tile_q0[tile];
+  const int t1 = min(t0 + 64, s1);
+  if (t1 <= t0) return;
+  const int C = B * n;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c_raw = blockIdx.x * 64 + lane;
+  const bool ok = c_raw < C;
+  const int c = ok ? c_raw : 0;
+  const int b = c / n, j = c - b * n;
+  const float br = gb[c], bi = gb[C + c], rt = rate[c];
+  const int tb = t0 + 16 * wave;
+  float av[16], bv[16], gv[16];
+  float LA = 0.f, L = 0.f;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    float zr[4], zi[4], uu[4], yy[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int t = tb + 4 * g + k;
+      const bool live = t < t1;
+      const A* zp = z + ((int64_t)b * T + t) * 2 * n + j;
+      zr[k] = live ? ldf<A>(zp) : 0.f;
+      zi[k] = live ? ldf<A>(zp + n) : 0.f;
+      uu[k] = live ? ldf<A>(u + (int64_t)t * C + c) : 0.f;
+      yy[k] = (MODE == 2 && live) ? ldf<A>(y + (int64_t)t * y_stride + c) : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const bool live = tb + 4 * g + k < t1;
+      const float la = live ? -rt * sigmoid_f(zr[k] + br) : 0.f;
+      const float a = exp_f(la);
+      const float bb = live ? sqrtf(one_minus_exp(2.f * la)) * sigmoid_f(zi[k] + bi) * uu[k] : 0.f;
+      av[4 * g + k] = a;
+      bv[4 * g + k] = bb;
+      gv[4 * g + k] = gelu_tanh_f(yy[k]);
+      LA += la;
+      L = a * L + bb;
+    }
+  }
+  sLA[wave][lane] = LA;
+  sL[wave][lane] = L;
+  __syncthreads();
+  float* wr = ws + ((int64_t)((t0 >> 6) + seq) * 2) * C + c;
   if (MODE == 1) {
-    wr[0] = LA;
-    wr[C] = S;
+    if (wave == 0 && ok) {
+      float la = sLA[0][lane], l = sL[0][lane];
+#pragma unroll
+      for (int v = 1; v < 4; ++v) {
+        l = exp_f(sLA[v][lane]) * l + sL[v][lane];
+        la += sLA[v][lane];
+      }
+      wr[0] = la;
+      wr[C] = l;
+    }
+  } else {
+    if (!ok) return;
+    float S = wr[C];
+    for (int v = 0; v < wave; ++v) S = exp_f(sLA[v][lane]) * S + sL[v][lane];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      S = av[i] * S + bv[i];
+      if (tb + i < t1) stf<O>(out + (int64_t)(tb + i) * C + c, S * gv[i]);
+    }
   }
 }
 
@@ -414,18 +481,20 @@ void launch_rm_rglru_scan(const void* z, const void* u, const void* y, bool bf16
   if (rows == 0 || seqs == 0) return;
   const int C = B * n, cb = (C + NT - 1) / NT;
   const bool blocks = num_tiles > 0 && ws != nullptr;
-#define RM_SCAN(MODE, grid_y)                                                                                                          \
-  RM_BF16(bf16, A, RM_BF16(out_bf16, O, hipLaunchKernelGGL((rglru_scan_kernel<A, O, MODE>), dim3(cb, grid_y), dim3(NT), 0, stream,     \
-                                                           (const A*)z, (const A*)u, (const A*)y, y_stride, gate_bias, rate, state,  \
-                                                           positions, qsl, state_slots, counts, rows, B, n, (O*)out, tile_seq,       \
-                                                           tile_q0, num_tiles, ws, blocks ? 1 : 0)))
-  RM_SCAN(0, seqs);
+#define RM_BLOCK(MODE)                                                                                                                 \
+  RM_BF16(bf16, A, RM_BF16(out_bf16, O, hipLaunchKernelGGL((rglru_block_kernel<A, O, MODE>), dim3((C + 63) / 64, num_tiles), dim3(NT), 0, \
+                                                           stream, (const A*)z, (const A*)u, (const A*)y, y_stride, gate_bias, rate,  \
+                                                           qsl, state_slots, counts, rows, B, n, (O*)out, tile_seq, tile_q0,         \
+                                                           num_tiles, ws)))
+  RM_BF16(bf16, A, RM_BF16(out_bf16, O, hipLaunchKernelGGL((rglru_scan_kernel<A, O>), dim3(cb, seqs), dim3(NT), 0, stream, (const A*)z,
+                                                           (const A*)u, (const A*)y, y_stride, gate_bias, rate, state, positions, qsl,
+                                                           state_slots, counts, rows, B, n, (O*)out, blocks ? 1 : 0)));
   if (blocks) {
-    RM_SCAN(1, num_tiles);
+    RM_BLOCK(1);
     hipLaunchKernelGGL(rglru_prefix_kernel, dim3(cb, seqs), dim3(NT), 0, stream, state, ws, positions, qsl, state_slots, counts, C);
-    RM_SCAN(2, num_tiles);
+    RM_BLOCK(2);
   }
-#undef RM_SCAN
+#undef RM_BLOCK
 }
 
 void launch_rm_latent_norm_cache(const void* proj, bool bf16, int64_t p_stride, int Q, const float* qw, const float* cw, float eps,
