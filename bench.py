@@ -12,6 +12,8 @@
     python bench.py --mixers --models mixtral,vibunex # side benchmark: Vibunex stacks beside Mixtral at equal layer sizes
     python bench.py --mixers --models mixtral,sevelorn-attention,rodelix-lightning,sevelorn-retention,llama,sevelorn
                                                       # side benchmark: Sevelorn stacks beside their closest families
+    python bench.py --mixers --models rodelix-lightning,sinilorn-recurrence,rodelix-latent_attention,sinilorn-latent,mixtral,sinilorn
+                                                      # side benchmark: Sinilorn stacks beside their closest families
 
 One rank per GPU.  ``--tp`` consecutive ranks form one tensor-parallel replica (``dp = gpus / tp`` replicas);
 every replica serves its share (round-robin, the router's stateless policy) of ONE global BurstGPT-like trace
