@@ -98,7 +98,7 @@ def sinilorn_raw(width, heads, kv, ffn, kinds):
     dense = {"kind": "dense", "ff": ffn}
     lat = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": width * 3 // 4, "scale": 192 ** -0.5,
            "mask": {"size": 1024},
-           "rot": {"base": 1000000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}
+           "rot": {"base": 1000000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "fast": 16.0, "slow": 2.0}}}
     mk = {
         "recurrence": {"type": "rglru", "mlp": dense, "mixer": {"blocks": width // 128, "conv": 4, "width": width}},
         "latent": {"type": "latent_attention", "mlp": moe, "mixer": lat},
