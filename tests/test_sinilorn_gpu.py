@@ -129,7 +129,7 @@ def test_block_scan_against_the_sequential_scan(tmp_path, monkeypatch):
     cases._check(blocks, cases.expect(cfg, W, toks), "float32", "block scan against the oracle")
 
 
-@pytest.mark.parametrize("T", [300, 9])
+@pytest.mark.parametrize("T", [300, 100, 9])
 def test_grouped_clamped_experts_against_the_row_kernels(T):
     """The clamped experts as grouped GEMMs (or, at decode size, weight streams) against the any-shape row kernels, same
     routing, identity experts among the picks."""
