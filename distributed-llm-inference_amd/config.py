@@ -43,13 +43,13 @@ class MixerSpec:
     vdim: int
     kv_heads: int = 0                   # attention: key / value heads
     scale: float = 1.0                  # multiplies q·k
-    window: int = 0                     # attention: a query sees itself and the window-1 tokens before it (0: all)
+    window: int = 0                     # attention, gated latent attention: a query sees itself and the window-1 tokens before it (0: all)
     kv_rank: int = 0                    # latent attention: size of the cached latent
     rot_dim: int = 0                    # latent attention: size of the rotated query / key part
     rot_base: float = 10000.0
     rot_dims: int = 0                   # leading entries of the rotated part that are actually rotated
     decay: tuple = ()                   # lightning: per-head state decay
-    rot_scaling: tuple = ()             # sink attention: (factor, original length, fast turns, slow turns) or ()
+    rot_scaling: tuple = ()             # sink / gated latent attention: (factor, original length, fast turns, slow turns) or ()
     lora: int = 0                       # time mix: rank of the decay projection
     parts: tuple = ()                   # parallel: the mixers run side by side (MixerSpec each)
     part_scales: tuple = ()             # parallel: weight of every part's output
@@ -59,8 +59,8 @@ class MixerSpec:
     top: int = 0                        # moe: experts per token
     router_scale: float = 1.0           # moe: multiplies the chosen experts' scores
     shared_ff: int = 0                  # moe: inner width of the expert every token takes (0: none)
-    kv_from: int = -1                   # gated attention: index of the layer whose cached keys / values this layer reads (-1: its own)
-    ff_act: str = "relu2"               # feed-forward activation: "relu2" | "gelu_tanh" (gated dense) | "silu" (gated experts)
+    kv_from: int = -1                   # gated (latent) attention: index of the layer whose cached rows this layer reads (-1: its own)
+    ff_act: str = "relu2"               # feed-forward activation: "relu2" | "gelu_tanh" / "silu" (gated) | "clamped" (gated experts)
     router: str = "sigmoid"             # moe: "sigmoid" (scores, not renormalised) | "softmax" (biased logits, softmax over the chosen)
                                         # | "softmax_all" (softmax over all logits, a choice bias, renormalised over the chosen)
     q_rank: int = 0                     # gated latent attention: size of the normed query latent

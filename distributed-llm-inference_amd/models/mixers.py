@@ -25,10 +25,17 @@ both, each through a sigmoid gate computed from its own input: ``x += m ¬∑ (g1 ‚
 * ``Retention`` ‚Äì linear attention with a per-head decay and no activation: rotated q / k, scaled keys, a ``[D, Dv]``
   fp32 state per head, per-head unit RMS and a silu gate behind it.
 
-``GatedDenseFF`` (``W_down (act(W_gate h) ‚äô W_up h)``) and ``SoftmaxRoutedFF`` (experts of that form behind a biased
-fp32 router, softmax over the chosen logits) are the feed-forwards of ``HyperLayer``, which keeps several copies of the
-fp32 stream: every sublayer reads a weighted sum of them through an RMS norm (the mixer also through a short causal
-convolution over time) and writes back through a mixing matrix.
+* ``GatedLinearRecurrence`` ‚Äì a per-channel recurrence ``S ‚Üê a ‚äô S + sqrt(1 - a¬≤) ‚äô i ‚äô u`` behind a short causal convolution:
+  decay and input gate from block-diagonal maps of ``u``, the fp32 state multiplied by a tanh-GELU branch;
+* ``GatedLatentAttention`` ‚Äì latent attention whose queries come from a normed latent too: half-split rotation with
+  optionally stretched frequencies, a sliding window, a per-head sink in the softmax denominator, an element-wise sigmoid
+  output gate; optionally without a key / value down-projection of its own, on another layer's cached latents.
+
+``GatedDenseFF`` (``W_down (act(W_gate h) ‚äô W_up h)``, optionally with biases), ``SoftmaxRoutedFF`` (experts of that form
+behind a biased fp32 router, softmax over the chosen logits) and ``ScoreRoutedFF`` (clamped gated experts and identity
+experts chosen by softmax scores plus a correction) are the feed-forwards of ``HyperLayer``, which keeps several copies of
+the fp32 stream: every sublayer reads a weighted sum of them through a norm (RMS with ``1 + w`` weights, or a layer norm
+without bias; the mixer optionally also through a short causal convolution over time) and writes back through a mixing matrix.
 
 ``MixerLayer`` wraps one of the first three (and an optional dense feed-forward) in the sandwich
 ``x += m ¬∑ norm_b(sublayer(norm(x)))`` with token shift in front of the mixer.  The residual stream ``x`` is
